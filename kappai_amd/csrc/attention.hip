@@ -316,7 +316,7 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
   const int g = h / (H / G);
   const int pos = row_pos[t];
   const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = kappai_first_key(pos, window);
   const T* qr = q + (size_t)t * q_stride + (size_t)h * d;
   for (int e = lane; e < d; e += WAVE) qs[e] = to_f32(qr[e]);
   __syncthreads();

@@ -165,8 +165,8 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
   const int pos_first = row_pos[r0], pos_last = pos_first + nr - 1;
   const bool row_ok = col < nr;
   const int my_pos = row_ok ? pos_first + col : -1;
-  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
-  const int lo_tile = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+  const int my_lo = kappai_first_key(my_pos, window);
+  const int lo_tile = kappai_first_key(pos_first, window);
 
   bf16x8_t qf[P_KS];
   {
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
   // page) plus an offset that a lane computes once.  The tiles at the window's lower edge and at
   // the diagonal take the general path.  Either way the loads of the next tile are issued
   // before the current one is worked on.
-  const int lo_last = (window > 0 && pos_last + 1 > window) ? pos_last + 1 - window : 0;
+  const int lo_last = kappai_first_key(pos_last, window);
   auto whole = [&](int kb) { return kb >= lo_last && kb + 31 <= pos_first; };
   const int k_lane = (col % 16) * HEAD_DIM + 8 * hh;       // + 16*ks
   const int v_lane = col * ps + 4 * hh;                    // + 32*mt*ps (+ 8)
@@ -472,18 +472,18 @@ __global__ __launch_bounds__(8 * WAVE) void attn_prefill_shared_kernel(
   const int pos_first = row_pos[r0], pos_last = pos_first + nr - 1;
   const bool row_ok = col < nr;
   const int my_pos = row_ok ? pos_first + col : -1;
-  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
-  const int lo_tile = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
-  const int lo_last = (window > 0 && pos_last + 1 > window) ? pos_last + 1 - window : 0;
+  const int my_lo = kappai_first_key(my_pos, window);
+  const int lo_tile = kappai_first_key(pos_first, window);
+  const int lo_last = kappai_first_key(pos_last, window);
   // the keys the block walks: from the first key of either tile to the last key of either
   int blk_first, blk_last;
   {
     const int ra = q_tiles[4 * t_a + 1], pa0 = row_pos[ra], pa1 = pa0 + q_tiles[4 * t_a + 2] - 1;
-    blk_first = (window > 0 && pa0 + 1 > window) ? pa0 + 1 - window : 0;
+    blk_first = kappai_first_key(pa0, window);
     blk_last = pa1;
     if (t_b >= 0) {
       const int rb = q_tiles[4 * t_b + 1], pb0 = row_pos[rb], pb1 = pb0 + q_tiles[4 * t_b + 2] - 1;
-      blk_first = min(blk_first, (window > 0 && pb0 + 1 > window) ? pb0 + 1 - window : 0);
+      blk_first = min(blk_first, kappai_first_key(pb0, window));
       blk_last = max(blk_last, pb1);
     }
   }
@@ -1158,7 +1158,7 @@ __device__ __forceinline__ void attn_decode_wave(
 // same number from the same table; splits past a row's keys do nothing and are not merged.
 #define D_TARGET_WAVES 2048
 __device__ __forceinline__ int keys_of_row(int pos, int window) {
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = kappai_first_key(pos, window);
   return pos + 1 - (lo / 32) * 32;
 }
 __device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_pos,
@@ -1212,7 +1212,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
                                              keys_per_split, n_splits)
                        : keys_per_split;
   const int* bt = block_tables + (size_t)seg * max_blocks;
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = kappai_first_key(pos, window);
   const int k_begin = (lo / 32) * 32 + split * kps;
   if (k_begin > pos) return;                                   // a split past the row's keys
   const int k_end = min(k_begin + kps, pos + 1);                // exclusive
@@ -1258,7 +1258,7 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
   const int col = lane % 16, kg = lane / 16;
   const int pos = row_pos[t];
   const int* bt = block_tables + (size_t)row_seg[t] * max_blocks;
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = kappai_first_key(pos, window);
   const int k_begin = (lo / 32) * 32;
   const int k_end = pos + 1;
   f32x4_t o[D_MT];

@@ -176,10 +176,10 @@ extern "C" int kappai_latent_store(const void* q, int q_stride, const void* kv, 
 #define HW_BN 64
 #define HW_BK 32
 
-template <typename T>
+template <typename T, typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(
     const T* __restrict__ x, int x_row, int x_head, const T* __restrict__ w, int n_out, int n_in,
-    T* __restrict__ y, int y_row, int y_head, int rows) {
+    TO* __restrict__ y, int y_row, int y_head, int rows) {
   __shared__ float xs[HW_BM][HW_BK + 1];
   __shared__ float ws[HW_BN][HW_BK + 1];
   const int h = blockIdx.z, m0 = blockIdx.x * HW_BM, n0 = blockIdx.y * HW_BN;
@@ -232,9 +232,10 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
 typedef __attribute__((ext_vector_type(8))) __bf16 hw_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float hw_f32x4_t;
 
+template <typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
     const bf16_t* __restrict__ x, int x_row, int x_head, const bf16_t* __restrict__ w, int n_out,
-    int n_in, bf16_t* __restrict__ y, int y_row, int y_head, int rows) {
+    int n_in, TO* __restrict__ y, int y_row, int y_head, int rows) {
   const int h = blockIdx.z, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int m0 = (blockIdx.x * (blockDim.x / WAVE) + wave) * 16, n0 = blockIdx.y * 64;
   if (m0 >= rows) return;
@@ -262,38 +263,122 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
                                                        0, 0, 0);
   }
   if (m0 + lr >= rows) return;
-  bf16_t* yr = y + (size_t)(m0 + lr) * y_row + (size_t)h * y_head;
+  TO* yr = y + (size_t)(m0 + lr) * y_row + (size_t)h * y_head;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int n = n0 + 16 * j + 4 * kq + v;
-      if (n < n_out) yr[n] = f32_to_bf16(acc[j][v]);
+      if (n < n_out) from_f32(yr + n, acc[j][v]);
     }
 }
 
+// out_f32: the results stay float32 although x and W are bfloat16 (what enters a recurrence).
 extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, const void* w, int H,
                                       int n_out, int n_in, void* y, int y_row, int y_head,
-                                      int rows, int is_bf16, hipStream_t stream) {
+                                      int rows, int is_bf16, int out_f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H < 1 || H > 65535 || n_out < 1 || n_in < 1) return (int)hipErrorInvalidValue;
   if (is_bf16 && n_in % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 &&
       ((uintptr_t)x | (uintptr_t)w) % 16 == 0 && (n_out + 63) / 64 <= 65535) {
     const int waves = rows <= 16 ? 1 : 4;
-    hipLaunchKernelGGL(headwise_linear_mfma_kernel,
-                       dim3((rows + 16 * waves - 1) / (16 * waves), (n_out + 63) / 64, H),
-                       dim3(waves * WAVE), 0, stream, (const bf16_t*)x, x_row, x_head,
-                       (const bf16_t*)w, n_out, n_in, (bf16_t*)y, y_row, y_head, rows);
+    const dim3 grid((rows + 16 * waves - 1) / (16 * waves), (n_out + 63) / 64, H);
+    if (out_f32)
+      hipLaunchKernelGGL(headwise_linear_mfma_kernel<float>, grid, dim3(waves * WAVE), 0, stream,
+                         (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in,
+                         (float*)y, y_row, y_head, rows);
+    else
+      hipLaunchKernelGGL(headwise_linear_mfma_kernel<bf16_t>, grid, dim3(waves * WAVE), 0, stream,
+                         (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in,
+                         (bf16_t*)y, y_row, y_head, rows);
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   dim3 grid((rows + HW_BM - 1) / HW_BM, (n_out + HW_BN - 1) / HW_BN, H);
   if (grid.y > 65535) return (int)hipErrorInvalidValue;
-  if (is_bf16)
-    hipLaunchKernelGGL(headwise_linear_kernel<bf16_t>, grid, dim3(256), 0, stream,
+  if (is_bf16 && out_f32)
+    hipLaunchKernelGGL((headwise_linear_kernel<bf16_t, float>), grid, dim3(256), 0, stream,
+                       (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in, (float*)y,
+                       y_row, y_head, rows);
+  else if (is_bf16)
+    hipLaunchKernelGGL((headwise_linear_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream,
                        (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in, (bf16_t*)y,
                        y_row, y_head, rows);
   else
-    hipLaunchKernelGGL(headwise_linear_kernel<float>, grid, dim3(256), 0, stream, (const float*)x,
-                       x_row, x_head, (const float*)w, n_out, n_in, (float*)y, y_row, y_head, rows);
+    hipLaunchKernelGGL((headwise_linear_kernel<float, float>), grid, dim3(256), 0, stream,
+                       (const float*)x, x_row, x_head, (const float*)w, n_out, n_in, (float*)y,
+                       y_row, y_head, rows);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// rotate_widen_store: grouped-query heads whose queries and keys (d) and values (dv) differ in
+// size, with a rotation over the first rot_dims places of every q and k head.  proj [T, H d +
+// G d (+ G dv)] as its product left it (biases added).  Queries leave as H heads of D (zeros
+// behind d); keys and values go to the pools as G heads of D.  values_are_keys: the projection
+// holds no values; a kv head's value is its key as projected, before the rotation (dv = d).
+// cos / sin [positions, rot_dims / 2] hold whatever factor the encoding puts on them.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(AP_THREADS) void rotate_widen_store_kernel(
+    const T* __restrict__ proj, int stride, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rot_dims, int rot_mode, int values_are_keys,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ row_pos,
+    const int* __restrict__ row_seg, const int* __restrict__ block_tables, int max_blocks, int H,
+    int G, int d, int dv, int D, int ps, T* __restrict__ q_out) {
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int pos = row_pos[t];
+  const T* row = proj + (size_t)t * stride;
+  const int nq = H * d, nk = G * d, half = rot_dims / 2;
+  const float* ct = cos_tab + (size_t)pos * half;
+  const float* st = sin_tab + (size_t)pos * half;
+  // place e of the head that starts at `head`: turned by the position, in float32
+  auto turned = [&](const T* head, int e) -> float {
+    const float x = to_f32(head[e]);
+    if (e >= rot_dims || rot_mode == 0) return x;
+    int j, partner;
+    bool first;
+    if (rot_mode == 1) { first = e < half; j = first ? e : e - half; partner = first ? e + half : e - half; }
+    else { first = (e & 1) == 0; j = e / 2; partner = e ^ 1; }
+    const float y = to_f32(head[partner]), c = ct[j], s = st[j];
+    return first ? x * c - y * s : x * c + y * s;
+  };
+  for (int i = tid; i < H * D; i += AP_THREADS) {
+    const int h = i / D, e = i % D;
+    from_f32(q_out + (size_t)t * H * D + i, e < d ? turned(row + h * d, e) : 0.f);
+  }
+  if (k_pool == nullptr) return;
+  const size_t page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
+  const int slot = pos % ps;
+  for (int i = tid; i < G * D; i += AP_THREADS) {
+    const int g = i / D, e = i % D;
+    const T* khead = row + nq + g * d;
+    float vv = 0.f;
+    if (e < dv) vv = values_are_keys ? to_f32(khead[e]) : to_f32(row[nq + nk + g * dv + e]);
+    from_f32(k_pool + ((page * G + g) * ps + slot) * D + e, e < d ? turned(khead, e) : 0.f);
+    from_f32(v_pool + ((page * G + g) * D + e) * ps + slot, vv);
+  }
+}
+
+extern "C" int kappai_rotate_widen_store(
+    const void* proj, int stride, const float* cos_tab, const float* sin_tab, int rot_dims,
+    int rot_mode, int values_are_keys, void* k_pool, void* v_pool, const int* row_pos,
+    const int* row_seg, const int* block_tables, int max_blocks, int T, int H, int G, int d,
+    int dv, int D, int ps, void* q_out, int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || d < 1 || dv < 1 || D < d || D < dv || ps < 1 || rot_dims < 0 ||
+      rot_dims > d || rot_dims % 2 || rot_mode < 0 || rot_mode > 2 ||
+      (values_are_keys && dv != d) || (rot_mode && rot_dims && (!cos_tab || !sin_tab)))
+    return (int)hipErrorInvalidValue;
+  if (rot_dims == 0) rot_mode = 0;
+  if (is_bf16)
+    hipLaunchKernelGGL(rotate_widen_store_kernel<bf16_t>, dim3(T), dim3(AP_THREADS), 0, stream,
+                       (const bf16_t*)proj, stride, cos_tab, sin_tab, rot_dims, rot_mode,
+                       values_are_keys, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, d, dv, D, ps, (bf16_t*)q_out);
+  else
+    hipLaunchKernelGGL(rotate_widen_store_kernel<float>, dim3(T), dim3(AP_THREADS), 0, stream,
+                       (const float*)proj, stride, cos_tab, sin_tab, rot_dims, rot_mode,
+                       values_are_keys, (float*)k_pool, (float*)v_pool, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, d, dv, D, ps, (float*)q_out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

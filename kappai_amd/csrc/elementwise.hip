@@ -154,6 +154,87 @@ extern "C" int kappai_output_norm_add(const void* a, int a_is_bf16, int a_parts,
 }
 
 // ---------------------------------------------------------------------------------------
+// Two sublayers' results side by side, made one update of the stream in float32:
+// out = scale_a * n_a(a) + scale_b * n_b(b), with n(y) = y / sqrt(mean(y^2) + eps) * w when a
+// weight is given and y itself when not.  a, b [T, D] in float32 or bfloat16 (one dtype); a block
+// a row, both rows in LDS between the sums of squares and the scaling.
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256) void pair_norm_sum_kernel(
+    const TA* __restrict__ a, float scale_a, const float* __restrict__ wa,
+    const TA* __restrict__ b, float scale_b, const float* __restrict__ wb, float eps, int D,
+    float* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) float ys[];
+  __shared__ float red[16];
+  const size_t at = (size_t)blockIdx.x * D;
+  float sa = 0.f, sb = 0.f;
+  for (int e = threadIdx.x; e < D; e += 256) {
+    const float x = to_f32(a[at + e]), y = to_f32(b[at + e]);
+    ys[e] = x;
+    ys[D + e] = y;
+    sa = fmaf(x, x, sa);
+    sb = fmaf(y, y, sb);
+  }
+  float fa = scale_a, fb = scale_b;
+  if (wa != nullptr) fa *= 1.0f / sqrtf(block_sum(sa, red) / (float)D + eps);
+  if (wb != nullptr) fb *= 1.0f / sqrtf(block_sum(sb, red) / (float)D + eps);
+  for (int e = threadIdx.x; e < D; e += 256) {
+    const float x = ys[e] * fa * (wa != nullptr ? wa[e] : 1.f);
+    const float y = ys[D + e] * fb * (wb != nullptr ? wb[e] : 1.f);
+    out[at + e] = x + y;
+  }
+}
+
+extern "C" int kappai_pair_norm_sum(const void* a, float scale_a, const float* wa, const void* b,
+                                    float scale_b, const float* wb, float eps, int T, int D,
+                                    float* out, int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (D < 1 || D > 7 * 1024) return (int)hipErrorInvalidValue;
+  const size_t lds = 2 * (size_t)D * sizeof(float);
+  if (is_bf16)
+    hipLaunchKernelGGL(pair_norm_sum_kernel<bf16_t>, dim3(T), dim3(256), lds, stream,
+                       (const bf16_t*)a, scale_a, wa, (const bf16_t*)b, scale_b, wb, eps, D, out);
+  else
+    hipLaunchKernelGGL(pair_norm_sum_kernel<float>, dim3(T), dim3(256), lds, stream,
+                       (const float*)a, scale_a, wa, (const float*)b, scale_b, wb, eps, D, out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// What a pass over a run of layers starts with: resid += delta (the update that the layer before
+// left pending; float32 or the compute dtype; may be null), then += again (rows of the same
+// shape, float32; may be null), then += row (one row [D] for all; may be null), in this order.
+// ---------------------------------------------------------------------------------------
+template <typename TD>
+__global__ __launch_bounds__(256) void stream_enter_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, const float* __restrict__ again,
+    const float* __restrict__ row, long n, int D) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float x = resid[i];
+  if (delta != nullptr) x += to_f32(delta[i]);
+  if (again != nullptr) x += again[i];
+  if (row != nullptr) x += row[i % D];
+  resid[i] = x;
+}
+
+extern "C" int kappai_stream_enter(float* resid, const void* delta, int delta_is_bf16,
+                                   const float* again, const float* row, int T, int D,
+                                   hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (D < 1) return (int)hipErrorInvalidValue;
+  const long n = (long)T * D;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (delta_is_bf16)
+    hipLaunchKernelGGL(stream_enter_kernel<bf16_t>, grid, dim3(256), 0, stream, resid,
+                       (const bf16_t*)delta, again, row, n, D);
+  else
+    hipLaunchKernelGGL(stream_enter_kernel<float>, grid, dim3(256), 0, stream, resid,
+                       (const float*)delta, again, row, n, D);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // tokens[dst_rows[i]] = chosen[src_idx[i]]: token ids that the last step's sampling kernels
 // left on the GPU go to their rows of this step's token table without a trip through the host.
 // ---------------------------------------------------------------------------------------
@@ -475,6 +556,31 @@ extern "C" int kappai_swiglu(const void* gu, void* act, int T, int F, int is_bf1
   else
     hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(threads), 0, stream,
                        (const float*)gu, (float*)act, F, n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// out[i] = f(in[i]) for one of a few functions: 0 tanh.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void unary_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n, int kind) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float x = to_f32(in[i]);
+  from_f32(out + i, kind == 0 ? tanhf(x) : x);
+}
+
+extern "C" int kappai_unary(const void* in, void* out, long n, int kind, int is_bf16,
+                            hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (kind != 0) return (int)hipErrorInvalidValue;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (is_bf16)
+    hipLaunchKernelGGL(unary_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                       (const bf16_t*)in, (bf16_t*)out, (size_t)n, kind);
+  else
+    hipLaunchKernelGGL(unary_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)in,
+                       (float*)out, (size_t)n, kind);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

@@ -3,6 +3,8 @@
 // decay per key channel:
 //   gated linear attention   S <- diag(a) S + k v^T                      o = S^T q
 //   gated delta rule         S <- diag(a) S; u = beta (v - S^T k); S <- S + k u^T;  o = S^T q
+//   bonus for the own token  o = (S + diag(u) k v^T)^T q;  S <- diag(a) S + k v^T   (the read-out
+//                            sees the state before the token and the token itself times u [H, d])
 // and what stands around them: the short causal convolution with SiLU on the projections, the
 // decays / unit vectors / step sizes in float32, and the per-head RMS norm with its gate.
 //
@@ -20,7 +22,8 @@ __device__ __forceinline__ float la_softplus(float x) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Short causal convolution per channel, then SiLU.  x [T, >= C] with a row stride, taps [C, n]
+// Short causal convolution per channel, then SiLU (act 1) or nothing (act 0), with an optional
+// bias [C] added before the activation.  x [T, >= C] with a row stride, taps [C, n]
 // (the last column meets the current token), state [slots, n - 1, C] float32: the last n - 1
 // inputs of the request, oldest first.  One thread a (row, channel) for the outputs; a second
 // kernel rewrites the state after the outputs are made.
@@ -30,7 +33,8 @@ __global__ __launch_bounds__(LA_THREADS) void conv_silu_kernel(
     const T* __restrict__ x, int x_stride, const float* __restrict__ taps, int n_taps,
     const float* __restrict__ state, const int* __restrict__ row_pos,
     const int* __restrict__ row_seg, const int* __restrict__ seg_start,
-    const int* __restrict__ seg_slot, int C, T* __restrict__ out) {
+    const int* __restrict__ seg_slot, int C, const float* __restrict__ bias, int act,
+    T* __restrict__ out) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * LA_THREADS + threadIdx.x;
   if (c >= C) return;
@@ -45,7 +49,8 @@ __global__ __launch_bounds__(LA_THREADS) void conv_silu_kernel(
     else v = st[(size_t)(n_taps - 1 - (back - (t - first))) * C + c];
     acc = fmaf(taps[(size_t)c * n_taps + j], v, acc);
   }
-  from_f32(out + (size_t)t * C + c, acc * la_sigmoid(acc));
+  if (bias != nullptr) acc += bias[c];
+  from_f32(out + (size_t)t * C + c, act ? acc * la_sigmoid(acc) : acc);
 }
 
 template <typename T>
@@ -73,14 +78,15 @@ __global__ __launch_bounds__(LA_THREADS) void conv_state_kernel(
 extern "C" int kappai_conv_silu(const void* x, int x_stride, const float* taps, int n_taps,
                                 float* state, const int* row_pos, const int* row_seg,
                                 const int* seg_start, const int* seg_pos0, const int* seg_slot,
-                                int T, int S, int C, void* out, int is_bf16, hipStream_t stream) {
+                                int T, int S, int C, const float* bias, int act, void* out,
+                                int is_bf16, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
   if (n_taps < 1 || n_taps > 17 || S > 65535 || C > 65535 * LA_THREADS) return (int)hipErrorInvalidValue;
   const int bx = (C + LA_THREADS - 1) / LA_THREADS;
   if (is_bf16) {
     hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, dim3(T, bx), dim3(LA_THREADS), 0, stream,
                        (const bf16_t*)x, x_stride, taps, n_taps, state, row_pos, row_seg,
-                       seg_start, seg_slot, C, (bf16_t*)out);
+                       seg_start, seg_slot, C, bias, act, (bf16_t*)out);
     if (n_taps > 1)
       hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(bx, S), dim3(LA_THREADS), 0, stream,
                          (const bf16_t*)x, x_stride, n_taps, state, seg_start, seg_pos0, seg_slot,
@@ -88,7 +94,7 @@ extern "C" int kappai_conv_silu(const void* x, int x_stride, const float* taps, 
   } else {
     hipLaunchKernelGGL(conv_silu_kernel<float>, dim3(T, bx), dim3(LA_THREADS), 0, stream,
                        (const float*)x, x_stride, taps, n_taps, state, row_pos, row_seg, seg_start,
-                       seg_slot, C, (float*)out);
+                       seg_slot, C, bias, act, (float*)out);
     if (n_taps > 1)
       hipLaunchKernelGGL(conv_state_kernel<float>, dim3(bx, S), dim3(LA_THREADS), 0, stream,
                          (const float*)x, x_stride, n_taps, state, seg_start, seg_pos0, seg_slot,
@@ -98,21 +104,107 @@ extern "C" int kappai_conv_silu(const void* x, int x_stride, const float* taps, 
 }
 
 // ---------------------------------------------------------------------------------------
+// Token shift: with h' the row before (the request's last row of the step before for a segment's
+// first row: state [slots, W] float32; zeros at position 0), out[m] = h + (h' - h) * mu[m] for
+// each of the n_mix rows of mu [n_mix, W], out [n_mix, T, W].  A thread a (row, channel); a
+// second kernel leaves every segment's last row as its state after the outputs are made.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(LA_THREADS) void token_shift_mix_kernel(
+    const T* __restrict__ h, int h_stride, const float* __restrict__ mu, int n_mix,
+    const float* __restrict__ state, const int* __restrict__ row_pos,
+    const int* __restrict__ row_seg, const int* __restrict__ seg_start,
+    const int* __restrict__ seg_slot, int rows, int W, T* __restrict__ out) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * LA_THREADS + threadIdx.x;
+  if (c >= W) return;
+  const int seg = row_seg[t];
+  const float cur = to_f32(h[(size_t)t * h_stride + c]);
+  float before = 0.f;
+  if (row_pos[t] > 0)
+    before = t > seg_start[seg] ? to_f32(h[(size_t)(t - 1) * h_stride + c])
+                                : state[(size_t)seg_slot[seg] * W + c];
+  const float diff = before - cur;
+  for (int m = 0; m < n_mix; ++m)
+    from_f32(out + ((size_t)m * rows + t) * W + c, fmaf(diff, mu[(size_t)m * W + c], cur));
+}
+
+template <typename T>
+__global__ __launch_bounds__(LA_THREADS) void token_shift_state_kernel(
+    const T* __restrict__ h, int h_stride, float* __restrict__ state,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_slot, int W) {
+  const int seg = blockIdx.y;
+  const int c = blockIdx.x * LA_THREADS + threadIdx.x;
+  if (c >= W) return;
+  const int last = seg_start[seg + 1] - 1;
+  if (last < seg_start[seg]) return;
+  state[(size_t)seg_slot[seg] * W + c] = to_f32(h[(size_t)last * h_stride + c]);
+}
+
+extern "C" int kappai_token_shift_mix(const void* h, int h_stride, const float* mu, int n_mix,
+                                      float* state, const int* row_pos, const int* row_seg,
+                                      const int* seg_start, const int* seg_slot, int T, int S,
+                                      int W, void* out, int is_bf16, hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (n_mix < 1 || W < 1 || S > 65535 || W > 65535 * LA_THREADS) return (int)hipErrorInvalidValue;
+  const int bx = (W + LA_THREADS - 1) / LA_THREADS;
+  if (is_bf16) {
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, dim3(T, bx), dim3(LA_THREADS), 0, stream,
+                       (const bf16_t*)h, h_stride, mu, n_mix, state, row_pos, row_seg, seg_start,
+                       seg_slot, T, W, (bf16_t*)out);
+    hipLaunchKernelGGL(token_shift_state_kernel<bf16_t>, dim3(bx, S), dim3(LA_THREADS), 0, stream,
+                       (const bf16_t*)h, h_stride, state, seg_start, seg_slot, W);
+  } else {
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(T, bx), dim3(LA_THREADS), 0, stream,
+                       (const float*)h, h_stride, mu, n_mix, state, row_pos, row_seg, seg_start,
+                       seg_slot, T, W, (float*)out);
+    hipLaunchKernelGGL(token_shift_state_kernel<float>, dim3(bx, S), dim3(LA_THREADS), 0, stream,
+                       (const float*)h, h_stride, state, seg_start, seg_slot, W);
+  }
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // What enters the recurrence, in float32: a wave a (row, head).
 //   qf, kf [T, Hk, d]   q and k (head h reads q/k head h / (H / Hk)), optionally made unit
 //                       vectors x / sqrt(sum x^2 + unit_eps); q also times q_scale
-//   af [T, H, d]        the decay exp(-rate[h] * softplus(sign * (z + z_bias)))
+//                       (act: silu of the projection as it is stored, rounded as it is stored)
+//   af [T, H, d]        the decay, by decay_kind: 0  exp(-rate[h] * softplus(sign * (z + z_bias)))
+//                                                 1  exp(-exp(z + z_bias))
+//                                                 2  rate[h] itself (z is not read)
 //   bf [T, H]           sigmoid(b) when b is given
+//   vf [T, H, dv]       silu(v), rounded as v is stored, when v is given
 // ---------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float la_stored_silu(float x) {
+  T r;
+  from_f32(&r, x * la_sigmoid(x));
+  return to_f32(r);
+}
+
 template <typename T>
 __global__ __launch_bounds__(WAVE) void recurrence_prep_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k, int k_stride,
     const T* __restrict__ z, int z_stride, const float* __restrict__ z_bias,
     const float* __restrict__ rate, float sign, const T* __restrict__ b, int b_stride, int H,
-    int Hk, int d, int unit, float unit_eps, float q_scale, float* __restrict__ qf,
-    float* __restrict__ kf, float* __restrict__ af, float* __restrict__ bf) {
+    int Hk, int d, int unit, float unit_eps, float q_scale, int act, int decay_kind,
+    const T* __restrict__ v, int v_stride, int dv, float* __restrict__ qf,
+    float* __restrict__ kf, float* __restrict__ af, float* __restrict__ bf,
+    float* __restrict__ vf) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  if (h < Hk) {
+  if (v != nullptr) {
+    const T* vr = v + (size_t)t * v_stride + (size_t)h * dv;
+    for (int e = lane; e < dv; e += WAVE)
+      vf[((size_t)t * H + h) * dv + e] = la_stored_silu<T>(to_f32(vr[e]));
+  }
+  if (h < Hk && act) {
+    const T* qr = q + (size_t)t * q_stride + (size_t)h * d;
+    const T* kr = k + (size_t)t * k_stride + (size_t)h * d;
+    for (int e = lane; e < d; e += WAVE) {
+      qf[((size_t)t * Hk + h) * d + e] = la_stored_silu<T>(to_f32(qr[e])) * q_scale;
+      kf[((size_t)t * Hk + h) * d + e] = la_stored_silu<T>(to_f32(kr[e]));
+    }
+  } else if (h < Hk) {
     const T* qr = q + (size_t)t * q_stride + (size_t)h * d;
     const T* kr = k + (size_t)t * k_stride + (size_t)h * d;
     float sq = 0.f, sk = 0.f;
@@ -131,11 +223,16 @@ __global__ __launch_bounds__(WAVE) void recurrence_prep_kernel(
       kf[((size_t)t * Hk + h) * d + e] = to_f32(kr[e]) * fk;
     }
   }
-  const T* zr = z + (size_t)t * z_stride + (size_t)h * d;
-  const float r = rate[h];
-  for (int e = lane; e < d; e += WAVE) {
-    const float zz = to_f32(zr[e]) + (z_bias ? z_bias[(size_t)h * d + e] : 0.f);
-    af[((size_t)t * H + h) * d + e] = expf(-r * la_softplus(sign * zz));
+  const float r = rate != nullptr ? rate[h] : 1.f;
+  if (decay_kind == 2) {
+    for (int e = lane; e < d; e += WAVE) af[((size_t)t * H + h) * d + e] = r;
+  } else {
+    const T* zr = z + (size_t)t * z_stride + (size_t)h * d;
+    for (int e = lane; e < d; e += WAVE) {
+      const float zz = to_f32(zr[e]) + (z_bias ? z_bias[(size_t)h * d + e] : 0.f);
+      af[((size_t)t * H + h) * d + e] =
+          decay_kind == 1 ? expf(-expf(zz)) : expf(-r * la_softplus(sign * zz));
+    }
   }
   if (b != nullptr && lane == 0)
     bf[(size_t)t * H + h] = la_sigmoid(to_f32(b[(size_t)t * b_stride + h]));
@@ -145,20 +242,26 @@ extern "C" int kappai_recurrence_prep(const void* q, int q_stride, const void* k
                                       const void* z, int z_stride, const float* z_bias,
                                       const float* rate, float sign, const void* b, int b_stride,
                                       int T, int H, int Hk, int d, int unit, float unit_eps,
-                                      float q_scale, float* qf, float* kf, float* af, float* bf,
-                                      int is_bf16, hipStream_t stream) {
+                                      float q_scale, int act, int decay_kind, const void* v,
+                                      int v_stride, int dv, float* qf, float* kf, float* af,
+                                      float* bf, float* vf, int is_bf16, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (H < 1 || Hk < 1 || H % Hk || H > 65535 || d < 1) return (int)hipErrorInvalidValue;
+  if (H < 1 || Hk < 1 || H % Hk || H > 65535 || d < 1 || decay_kind < 0 || decay_kind > 2 ||
+      (decay_kind != 2 && z == nullptr) || (decay_kind != 1 && rate == nullptr) ||
+      (act && unit) || (v != nullptr && (vf == nullptr || dv < 1)))
+    return (int)hipErrorInvalidValue;
   if (is_bf16)
     hipLaunchKernelGGL(recurrence_prep_kernel<bf16_t>, dim3(T, H), dim3(WAVE), 0, stream,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)z,
                        z_stride, z_bias, rate, sign, (const bf16_t*)b, b_stride, H, Hk, d, unit,
-                       unit_eps, q_scale, qf, kf, af, bf);
+                       unit_eps, q_scale, act, decay_kind, (const bf16_t*)v, v_stride, dv, qf, kf,
+                       af, bf, vf);
   else
     hipLaunchKernelGGL(recurrence_prep_kernel<float>, dim3(T, H), dim3(WAVE), 0, stream,
                        (const float*)q, q_stride, (const float*)k, k_stride, (const float*)z,
                        z_stride, z_bias, rate, sign, (const float*)b, b_stride, H, Hk, d, unit,
-                       unit_eps, q_scale, qf, kf, af, bf);
+                       unit_eps, q_scale, act, decay_kind, (const float*)v, v_stride, dv, qf, kf,
+                       af, bf, vf);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -169,7 +272,7 @@ extern "C" int kappai_recurrence_prep(const void* q, int q_stride, const void* k
 // decay (no two on one LDS bank).  Few rows a lane, because a wave alone on its SIMD issues an
 // instruction only every ten cycles or so: the walk along the tokens is as fast as a wave's
 // instructions per token are few, and idle SIMDs are there to take more waves.  These lanes
-// are neighbours, and their partial dot products meet by data-parallel moves.  DELTA: the delta rule (needs beta), else the plain gated sum.
+// are neighbours, and their partial dot products meet by data-parallel moves.  MODE 0: the plain gated sum; 1: the delta rule (needs beta); 2: the bonus for the own token.
 // In memory a head's matrix lies column by column: state [slots, H, dv, d], so that a lane's rows
 // are consecutive and a wave's columns one stretch.
 //
@@ -242,12 +345,19 @@ __device__ __forceinline__ void la_store_rows(float* __restrict__ st, int s, int
 // One token: S, the lane's rows of q, k and the decay, the column's v, the head's beta.  The dot
 // products are summed in four strands (rows r, r + 4, ...) that meet at the end: four short
 // chains of dependent operations instead of one long one.
-template <int KS, int R, bool DELTA>
+template <int KS, int R, int MODE>
 __device__ __forceinline__ float la_token(float (&S)[R], const float (&qc)[R],
                                           const float (&kc)[R], const float (&ac)[R],
-                                          float vc, float bc) {
+                                          const float (&uc)[R], float vc, float bc) {
   float o[4] = {0.f, 0.f, 0.f, 0.f};
-  if (DELTA) {
+  if (MODE == 2) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float kv = kc[r] * vc;
+      o[r % 4] = fmaf(fmaf(uc[r], kv, S[r]), qc[r], o[r % 4]);
+      S[r] = fmaf(ac[r], S[r], kv);
+    }
+  } else if (MODE == 1) {
     float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -276,7 +386,7 @@ __device__ __forceinline__ float la_token(float (&S)[R], const float (&qc)[R],
 // and the decay (piece i = tid + j * threads: token i / (d / 4), floats 4 (i % (d / 4)) ..), and
 // up to LA_MAX_CHUNK values of v.
 #define LA_QS 4
-template <int KS, int R, bool DELTA, typename TV>
+template <int KS, int R, int MODE, typename TV>
 __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_kernel(
     const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ af,
     const float* __restrict__ bf, const TV* __restrict__ v, int v_stride,
@@ -297,6 +407,10 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
   float* st = state + (((size_t)seg_slot[seg] * H + h) * dv + cc) * d;
   float S[R];
   la_load_rows<KS, R>(st, s, d, seg_pos0[seg] > 0, S);
+  float uc[R];      // MODE 2: the lane's rows of the head's bonus, which `bf` then holds [H, d]
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    uc[r] = MODE == 2 && la_row<KS>(s, r) < d ? bf[(size_t)h * d + la_row<KS>(s, r)] : 0.f;
 
   // the thread's places
   const int g4 = d / 4;
@@ -331,7 +445,7 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
         const int tt = (tid + j * nthr) >> nwc_log2;
         if (tt < n) sv[j] = to_f32(v[(size_t)(t0 + tt) * v_stride + (size_t)h * dv + v_col]);
       }
-    if (DELTA && tid < n) sb = bf[(size_t)(t0 + tid) * H + h];
+    if (MODE == 1 && tid < n) sb = bf[(size_t)(t0 + tid) * H + h];
   };
   // ... and from the registers to LDS
   auto put = [&](int n) {
@@ -348,7 +462,7 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
         const int i = tid + j * nthr, tt = i >> nwc_log2;
         if (tt < n) sh_scan[tt * rec + 3 * DP + (i & (NWC - 1))] = sv[j];
       }
-    if (DELTA && tid < n) sh_scan[tid * rec + 3 * DP + NWC] = sb;
+    if (MODE == 1 && tid < n) sh_scan[tid * rec + 3 * DP + NWC] = sb;
   };
   // a token's values for this lane out of LDS
   auto read = [&](int tt, float (&q_)[R], float (&k_)[R], float (&a_)[R], float& v_,
@@ -390,15 +504,15 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
     int tt = 0;
     for (; tt + 1 < n; tt += 2) {
       read(tt + 1, q1, k1, a1, v1, b1);
-      const float o0 = la_token<KS, R, DELTA>(S, q0, k0, a0, v0, b0);
+      const float o0 = la_token<KS, R, MODE>(S, q0, k0, a0, uc, v0, b0);
       if (writes) op[0] = o0;
       read(min(tt + 2, tb - 1), q0, k0, a0, v0, b0);
-      const float o1 = la_token<KS, R, DELTA>(S, q1, k1, a1, v1, b1);
+      const float o1 = la_token<KS, R, MODE>(S, q1, k1, a1, uc, v1, b1);
       if (writes) op[ostep] = o1;
       op += 2 * ostep;
     }
     if (tt < n) {
-      const float o0 = la_token<KS, R, DELTA>(S, q0, k0, a0, v0, b0);
+      const float o0 = la_token<KS, R, MODE>(S, q0, k0, a0, uc, v0, b0);
       if (writes) op[0] = o0;
     }
     __syncthreads();
@@ -408,7 +522,7 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
   if (col_ok) la_store_rows<KS, R>(st, s, d, S);
 }
 
-template <int KS, int R, bool DELTA, typename TV>
+template <int KS, int R, int MODE, typename TV>
 __global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
     const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ af,
     const float* __restrict__ bf, const TV* __restrict__ v, int v_stride,
@@ -425,6 +539,10 @@ __global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
   float* st = state + (((size_t)seg_slot[seg] * H + h) * dv + cc) * d;
   float S[R];
   la_load_rows<KS, R>(st, s, d, seg_pos0[seg] > 0, S);
+  float uc[R];      // MODE 2: the lane's rows of the head's bonus, which `bf` then holds [H, d]
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    uc[r] = MODE == 2 && la_row<KS>(s, r) < d ? bf[(size_t)h * d + la_row<KS>(s, r)] : 0.f;
 
   float qn[R], kn[R], an[R], vn = 0.f, bn = 0.f;
   auto fetch = [&](int t) {
@@ -440,7 +558,7 @@ __global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
       an[r] = ok ? ar[row] : 0.f;
     }
     vn = to_f32(v[(size_t)t * v_stride + (size_t)h * dv + cc]);
-    if (DELTA) bn = bf[(size_t)t * H + h];
+    if (MODE == 1) bn = bf[(size_t)t * H + h];
   };
   if (first < last) fetch(first);
   for (int t = first; t < last; ++t) {
@@ -449,7 +567,7 @@ __global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
     for (int r = 0; r < R; ++r) { qc[r] = qn[r]; kc[r] = kn[r]; ac[r] = an[r]; }
     const float vc = vn, bc = bn;
     if (t + 1 < last) fetch(t + 1);
-    const float o = la_token<KS, R, DELTA>(S, qc, kc, ac, vc, bc);
+    const float o = la_token<KS, R, MODE>(S, qc, kc, ac, uc, vc, bc);
     if (s == 0 && col_ok) out[(size_t)t * H * dv + (size_t)h * dv + c] = o;
   }
   if (col_ok) la_store_rows<KS, R>(st, s, d, S);
@@ -475,7 +593,7 @@ static LaBlockShape la_block_shape(int ks, int r, int H, int S, int T, int d, in
   return LaBlockShape{nw, tb, lg, rec};
 }
 
-template <int KS, int R, bool DELTA, typename TV>
+template <int KS, int R, int MODE, typename TV>
 static void scan_launch_typed(const float* qf, const float* kf, const float* af, const float* bf,
                               const TV* v, int v_stride, float* state, const int* seg_start,
                               const int* seg_pos0, const int* seg_slot, int T, int S, int H,
@@ -483,31 +601,31 @@ static void scan_launch_typed(const float* qf, const float* kf, const float* af,
   constexpr int COLS = WAVE / KS;
   const LaBlockShape b = la_block_shape(KS, R, H, S, T, d, dv);
   if (form == 1 || b.tb < 1) {
-    hipLaunchKernelGGL((matrix_state_scan_wave_kernel<KS, R, DELTA, TV>),
+    hipLaunchKernelGGL((matrix_state_scan_wave_kernel<KS, R, MODE, TV>),
                        dim3((dv + COLS - 1) / COLS, H, S), dim3(WAVE), 0, stream, qf, kf, af, bf,
                        v, v_stride, state, seg_start, seg_pos0, seg_slot, H, Hk, d, dv, out);
     return;
   }
   const int nwc = b.nw * COLS;
-  hipLaunchKernelGGL((matrix_state_scan_block_kernel<KS, R, DELTA, TV>),
+  hipLaunchKernelGGL((matrix_state_scan_block_kernel<KS, R, MODE, TV>),
                      dim3((dv + nwc - 1) / nwc, H, S), dim3(b.nw * WAVE),
                      (size_t)b.tb * b.rec * sizeof(float), stream, qf, kf, af, bf, v, v_stride,
                      state, seg_start, seg_pos0, seg_slot, H, Hk, d, dv, b.tb, b.rec, b.nwc_log2,
                      out);
 }
 
-template <int KS, int R, bool DELTA>
+template <int KS, int R, int MODE>
 static void scan_launch(const float* qf, const float* kf, const float* af, const float* bf,
                         const void* v, int v_stride, int v_is_bf16, float* state,
                         const int* seg_start, const int* seg_pos0, const int* seg_slot, int T,
                         int S, int H, int Hk, int d, int dv, int form, float* out,
                         hipStream_t stream) {
   if (v_is_bf16)
-    scan_launch_typed<KS, R, DELTA, bf16_t>(qf, kf, af, bf, (const bf16_t*)v, v_stride, state,
+    scan_launch_typed<KS, R, MODE, bf16_t>(qf, kf, af, bf, (const bf16_t*)v, v_stride, state,
                                          seg_start, seg_pos0, seg_slot, T, S, H, Hk, d, dv, form,
                                          out, stream);
   else
-    scan_launch_typed<KS, R, DELTA, float>(qf, kf, af, bf, (const float*)v, v_stride, state,
+    scan_launch_typed<KS, R, MODE, float>(qf, kf, af, bf, (const float*)v, v_stride, state,
                                         seg_start, seg_pos0, seg_slot, T, S, H, Hk, d, dv, form,
                                         out, stream);
 }
@@ -517,13 +635,15 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
                                         const float* bf, const void* v, int v_stride,
                                         int v_is_bf16, float* state, const int* seg_start,
                                         const int* seg_pos0, const int* seg_slot, int T, int S,
-                                        int H, int Hk, int d, int dv, int delta, int form,
+                                        int H, int Hk, int d, int dv, int mode, int form,
                                         float* out, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
   if (H < 1 || Hk < 1 || H % Hk || H > 65535 || S > 65535 || d < 1 || d > 64 * 16 || dv < 1 ||
-      form < 0 || form > 2)
+      form < 0 || form > 2 || mode < 0 || mode > 2)
     return (int)hipErrorInvalidValue;
-  if (delta && bf == nullptr) return (int)hipErrorInvalidValue;
+  // mode 1 (delta rule): bf = beta [T, H]; mode 2 (bonus): bf = the bonus [H, d], H == Hk
+  if (mode && bf == nullptr) return (int)hipErrorInvalidValue;
+  if (mode == 2 && H != Hk) return (int)hipErrorInvalidValue;
   // eight rows a lane; sixteen for the key sizes that 64 lanes of eight do not hold
   const int r = d <= 64 * 8 ? 8 : 16;
   int ks = 1;
@@ -531,11 +651,14 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
   if (form == 2 && la_block_shape(ks, r, H, S, T, d, dv).tb < 1) return (int)hipErrorInvalidValue;
 #define LA_CASE(KS_, R_)                                                                          \
   case KS_ * 100 + R_:                                                                                    \
-    if (delta)                                                                                  \
-      scan_launch<KS_, R_, true>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
+    if (mode == 1)                                                                              \
+      scan_launch<KS_, R_, 1>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
+                             seg_slot, T, S, H, Hk, d, dv, form, out, stream);                     \
+    else if (mode == 2)                                                                         \
+      scan_launch<KS_, R_, 2>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
                              seg_slot, T, S, H, Hk, d, dv, form, out, stream);                     \
     else                                                                                        \
-      scan_launch<KS_, R_, false>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start,         \
+      scan_launch<KS_, R_, 0>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start,         \
                               seg_pos0, seg_slot, T, S, H, Hk, d, dv, form, out, stream);          \
     break;
   switch (ks * 100 + r) {
@@ -550,12 +673,15 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
 // ---------------------------------------------------------------------------------------
 // Per head: o / sqrt(mean(o^2) + eps) * weight[dv] * gate, gate = silu(g) (kind 0) or sigmoid(g)
 // (kind 1) of the projection g [T, >= H dv] with a row stride.  A wave a (row, head).
+// weight_stride: 0 when the heads share one weight [dv], dv when each has its own [H, dv].
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(
     const float* __restrict__ o, const float* __restrict__ weight, float eps,
-    const T* __restrict__ g, int g_stride, int gate_kind, int H, int dv, T* __restrict__ out) {
+    const T* __restrict__ g, int g_stride, int gate_kind, int H, int dv, int weight_stride,
+    T* __restrict__ out) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  weight += (size_t)h * weight_stride;
   const float* orow = o + ((size_t)t * H + h) * dv;
   float ss = 0.f;
   for (int e = lane; e < dv; e += WAVE) ss = fmaf(orow[e], orow[e], ss);
@@ -569,16 +695,17 @@ __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(
 }
 
 extern "C" int kappai_head_norm_gate(const float* o, const float* weight, float eps, const void* g,
-                                     int g_stride, int gate_kind, int T, int H, int dv, void* out,
-                                     int is_bf16, hipStream_t stream) {
+                                     int g_stride, int gate_kind, int T, int H, int dv,
+                                     int weight_stride, void* out, int is_bf16,
+                                     hipStream_t stream) {
   if (T <= 0) return 0;
   if (H < 1 || H > 65535 || dv < 1 || gate_kind < 0 || gate_kind > 1)
     return (int)hipErrorInvalidValue;
   if (is_bf16)
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(T, H), dim3(WAVE), 0, stream, o, weight,
-                       eps, (const bf16_t*)g, g_stride, gate_kind, H, dv, (bf16_t*)out);
+                       eps, (const bf16_t*)g, g_stride, gate_kind, H, dv, weight_stride, (bf16_t*)out);
   else
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(T, H), dim3(WAVE), 0, stream, o, weight,
-                       eps, (const float*)g, g_stride, gate_kind, H, dv, (float*)out);
+                       eps, (const float*)g, g_stride, gate_kind, H, dv, weight_stride, (float*)out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -1,8 +1,16 @@
-// minGRU: S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, z = sigmoid(pz), c = pu + 1/2 where
-// pu >= 0 and sigmoid(pu) below, y_t = S_t * silu(pg).  The projections [T, 3W] = (pz | pu | pg)
-// come with their biases added, in float32 or as the bfloat16 a product stored; gates, candidates
-// and the state are float32; the state lives in a slot per request [slots, W] and a segment that
-// starts at position 0 starts from zero.
+// Recurrences with one number of state a channel, S_t = a_t S_(t-1) + b_t, whose a_t and b_t read
+// the current token only.  Gates, candidates and the state are float32; the state lives in a slot
+// per request [slots, W] and a segment that starts at position 0 starts from zero.
+//
+// minGRU (KIND 0): a = 1 - z, b = z c with z = sigmoid(pz), c = pu + 1/2 where pu >= 0 and
+// sigmoid(pu) below, y_t = S_t * silu(pg).  The projections [T, 3W] = (pz | pu | pg) come with
+// their biases added, in float32 or as the bfloat16 a product stored.
+//
+// Real-gated unit (KIND 1): a = exp(-rate * sigmoid(gr) * sp[c]), b = sqrt(1 - a^2) * sigmoid(gi)
+// * u, y_t = S_t * gelu_tanh(py): gr | gi [T, 2W] float32 are the gates before their sigmoid, u
+// [T, W] the channel's input (a convolution's result, as stored), py the other branch's projection
+// (a view with a row stride, as stored), sp [W] float32 (softplus of the channel's parameter);
+// gate_bias [2W] is added to gr | gi before the sigmoid.
 #include "common.h"
 
 #define MG_THREADS 256
@@ -16,11 +24,46 @@ __device__ __forceinline__ void mingru_gates(float pz, float pu, float& a, float
   b = z * c;
 }
 
+// What a scan reads.  KIND 0 uses proj alone.
+template <typename TP>
+struct scan_in {
+  const TP* proj;          // KIND 0: [T, 3W]; KIND 1: the gated branch, rows `y_stride` apart
+  const float* gates;      // KIND 1: [T, 2W]
+  const float* gate_bias;  // KIND 1: [2W], added to the gates before their sigmoid
+  const TP* u;             // KIND 1: [T, W]
+  const float* sp;         // KIND 1: [W]
+  float rate;              // KIND 1
+  int y_stride;            // KIND 1
+};
+
+// a, b of row t and channel c, and (OUT) the factor on the state that makes the output
+template <int KIND, bool OUT, typename TP>
+__device__ __forceinline__ void scan_terms(const scan_in<TP>& in, int W, int t, int c, float& a,
+                                           float& b, float& g) {
+  if (KIND == 0) {
+    const TP* p = in.proj + (size_t)t * 3 * W + c;
+    mingru_gates(to_f32(p[0]), to_f32(p[W]), a, b);
+    if (OUT) {
+      const float pg = to_f32(p[2 * W]);
+      g = pg * sigmoid_f(pg);
+    }
+  } else {
+    const float* gp = in.gates + (size_t)t * 2 * W + c;
+    const float uu = to_f32(in.u[(size_t)t * W + c]);
+    a = expf(-in.rate * sigmoid_f(gp[0] + in.gate_bias[c]) * in.sp[c]);
+    b = sqrtf(fmaxf(1.0f - a * a, 0.f)) * sigmoid_f(gp[W] + in.gate_bias[W + c]) * uu;
+    if (OUT) {
+      const float z = to_f32(in.proj[(size_t)t * in.y_stride + c]);
+      g = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    }
+  }
+}
+
 // One thread a (segment, channel), walking the segment's rows in order: what a step of few rows
 // a request runs (decoding, short portions).
-template <typename TP, typename TO>
+template <int KIND, typename TP, typename TO>
 __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
-    const TP* __restrict__ proj, float* __restrict__ state, const int* __restrict__ seg_start,
+    const scan_in<TP> in, float* __restrict__ state, const int* __restrict__ seg_start,
     const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot, int W,
     TO* __restrict__ out) {
   const int seg = blockIdx.y;
@@ -30,12 +73,10 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
   float* st = state + (size_t)seg_slot[seg] * W + c;
   float S = seg_pos0[seg] > 0 ? *st : 0.f;
   for (int t = first; t < last; ++t) {
-    const TP* p = proj + (size_t)t * 3 * W + c;
-    float a, b;
-    mingru_gates(to_f32(p[0]), to_f32(p[W]), a, b);
+    float a, b, g;
+    scan_terms<KIND, true>(in, W, t, c, a, b, g);
     S = fmaf(a, S, b);
-    const float g = to_f32(p[2 * W]);
-    from_f32(out + (size_t)t * W + c, S * (g * sigmoid_f(g)));
+    from_f32(out + (size_t)t * W + c, S * g);
   }
   *st = S;
 }
@@ -47,9 +88,9 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
 // every chunk's start in place of them.  Pass 3: every chunk walks its rows from that state and
 // writes the outputs.  The state a row sees is the same sum of products whatever the chunks are,
 // up to rounding.
-template <typename TP>
+template <int KIND, typename TP>
 __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_sums_kernel(
-    const TP* __restrict__ proj, const int* __restrict__ chunks, int W,
+    const scan_in<TP> in, const int* __restrict__ chunks, int W,
     float* __restrict__ carry) {
   const int ch = blockIdx.y;
   const int c = blockIdx.x * MG_THREADS + threadIdx.x;
@@ -58,20 +99,15 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_sums_kernel(
   float A = 1.f, B = 0.f;
   // (four rows' loads at a time, so that they do not wait for one another)
   for (int t0 = first; t0 < first + n; t0 += 4) {
-    float pz[4], pu[4];
+    float a[4], b[4], g;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const TP* p = proj + (size_t)min(t0 + i, first + n - 1) * 3 * W + c;
-      pz[i] = to_f32(p[0]);
-      pu[i] = to_f32(p[W]);
-    }
+    for (int i = 0; i < 4; ++i)
+      scan_terms<KIND, false>(in, W, min(t0 + i, first + n - 1), c, a[i], b[i], g);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (t0 + i >= first + n) break;
-      float a, b;
-      mingru_gates(pz[i], pu[i], a, b);
-      A *= a;
-      B = fmaf(a, B, b);
+      A *= a[i];
+      B = fmaf(a[i], B, b[i]);
     }
   }
   carry[((size_t)ch * 3) * W + c] = A;
@@ -106,9 +142,9 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_carry_kernel(
   *st = S;
 }
 
-template <typename TP, typename TO>
+template <int KIND, typename TP, typename TO>
 __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_out_kernel(
-    const TP* __restrict__ proj, const int* __restrict__ chunks, int W,
+    const scan_in<TP> in, const int* __restrict__ chunks, int W,
     const float* __restrict__ carry, TO* __restrict__ out) {
   const int ch = blockIdx.y;
   const int c = blockIdx.x * MG_THREADS + threadIdx.x;
@@ -116,44 +152,37 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_out_kernel(
   const int first = chunks[3 * ch + 1], n = chunks[3 * ch + 2];
   float S = carry[((size_t)ch * 3 + 2) * W + c];
   for (int t0 = first; t0 < first + n; t0 += 4) {
-    float pz[4], pu[4], pg[4];
+    float a[4], b[4], g[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const TP* p = proj + (size_t)min(t0 + i, first + n - 1) * 3 * W + c;
-      pz[i] = to_f32(p[0]);
-      pu[i] = to_f32(p[W]);
-      pg[i] = to_f32(p[2 * W]);
-    }
+    for (int i = 0; i < 4; ++i)
+      scan_terms<KIND, true>(in, W, min(t0 + i, first + n - 1), c, a[i], b[i], g[i]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (t0 + i >= first + n) break;
-      float a, b;
-      mingru_gates(pz[i], pu[i], a, b);
-      S = fmaf(a, S, b);
-      from_f32(out + (size_t)(t0 + i) * W + c, S * (pg[i] * sigmoid_f(pg[i])));
+      S = fmaf(a[i], S, b[i]);
+      from_f32(out + (size_t)(t0 + i) * W + c, S * g[i]);
     }
   }
 }
 
-template <typename TP, typename TO>
-static void mingru_launch(const void* proj_v, float* state, const int* seg_start,
-                          const int* seg_pos0, const int* seg_slot, int S, int W, const int* chunks,
-                          const int* seg_chunk0, int n_chunks, float* carry, void* out_v,
-                          hipStream_t stream) {
-  const TP* proj = (const TP*)proj_v;
+template <int KIND, typename TP, typename TO>
+static void scan_launch(const scan_in<TP>& in, float* state, const int* seg_start,
+                        const int* seg_pos0, const int* seg_slot, int S, int W, const int* chunks,
+                        const int* seg_chunk0, int n_chunks, float* carry, void* out_v,
+                        hipStream_t stream) {
   TO* out = (TO*)out_v;
   const int bx = (W + MG_THREADS - 1) / MG_THREADS;
   if (chunks == nullptr) {
-    hipLaunchKernelGGL((mingru_scan_rows_kernel<TP, TO>), dim3(bx, S), dim3(MG_THREADS), 0, stream,
-                       proj, state, seg_start, seg_pos0, seg_slot, W, out);
+    hipLaunchKernelGGL((mingru_scan_rows_kernel<KIND, TP, TO>), dim3(bx, S), dim3(MG_THREADS), 0,
+                       stream, in, state, seg_start, seg_pos0, seg_slot, W, out);
     return;
   }
-  hipLaunchKernelGGL(mingru_chunk_sums_kernel<TP>, dim3(bx, n_chunks), dim3(MG_THREADS), 0, stream,
-                     proj, chunks, W, carry);
+  hipLaunchKernelGGL((mingru_chunk_sums_kernel<KIND, TP>), dim3(bx, n_chunks), dim3(MG_THREADS), 0,
+                     stream, in, chunks, W, carry);
   hipLaunchKernelGGL(mingru_chunk_carry_kernel, dim3(bx, S), dim3(MG_THREADS), 0, stream,
                      seg_chunk0, seg_pos0, seg_slot, W, carry, state);
-  hipLaunchKernelGGL((mingru_chunk_out_kernel<TP, TO>), dim3(bx, n_chunks), dim3(MG_THREADS), 0,
-                     stream, proj, chunks, W, carry, out);
+  hipLaunchKernelGGL((mingru_chunk_out_kernel<KIND, TP, TO>), dim3(bx, n_chunks),
+                     dim3(MG_THREADS), 0, stream, in, chunks, W, carry, out);
 }
 
 // `chunks` [n_chunks, 3] = (segment, first row, rows) and `seg_chunk0` [S + 1] (first chunk of
@@ -171,13 +200,45 @@ extern "C" int kappai_mingru_scan(const void* proj, int proj_is_bf16, float* sta
     return (int)hipErrorInvalidValue;
   if (proj_is_bf16 && !out_is_bf16) return (int)hipErrorInvalidValue;
   if (proj_is_bf16)
-    mingru_launch<bf16_t, bf16_t>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
-                                  seg_chunk0, n_chunks, carry, out, stream);
+    scan_launch<0, bf16_t, bf16_t>(scan_in<bf16_t>{(const bf16_t*)proj, nullptr, nullptr, nullptr, nullptr,
+                                                   0.f, 0},
+                                   state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
+                                   n_chunks, carry, out, stream);
   else if (out_is_bf16)
-    mingru_launch<float, bf16_t>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
-                                 seg_chunk0, n_chunks, carry, out, stream);
+    scan_launch<0, float, bf16_t>(scan_in<float>{(const float*)proj, nullptr, nullptr, nullptr, nullptr,
+                                                 0.f, 0},
+                                  state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
+                                  n_chunks, carry, out, stream);
   else
-    mingru_launch<float, float>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
-                                seg_chunk0, n_chunks, carry, out, stream);
+    scan_launch<0, float, float>(scan_in<float>{(const float*)proj, nullptr, nullptr, nullptr, nullptr,
+                                                0.f, 0},
+                                 state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
+                                 n_chunks, carry, out, stream);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// The real-gated unit through the same kernels; `out` is stored as `u` and `y` are.
+extern "C" int kappai_gated_unit_scan(const float* gates, const float* gate_bias, const void* u,
+                                      const void* y,
+                                      int y_stride, const float* sp, float rate, int is_bf16,
+                                      float* state, const int* seg_start, const int* seg_pos0,
+                                      const int* seg_slot, int T, int S, int W, const int* chunks,
+                                      const int* seg_chunk0, int n_chunks, float* carry, void* out,
+                                      hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (S > 65535 || n_chunks > 65535 || W < 1 || y_stride < W || gate_bias == nullptr)
+    return (int)hipErrorInvalidValue;
+  if (chunks != nullptr && (n_chunks <= 0 || carry == nullptr || seg_chunk0 == nullptr))
+    return (int)hipErrorInvalidValue;
+  if (is_bf16)
+    scan_launch<1, bf16_t, bf16_t>(scan_in<bf16_t>{(const bf16_t*)y, gates, gate_bias, (const bf16_t*)u, sp,
+                                                   rate, y_stride},
+                                   state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
+                                   n_chunks, carry, out, stream);
+  else
+    scan_launch<1, float, float>(scan_in<float>{(const float*)y, gates, gate_bias, (const float*)u, sp, rate,
+                                                y_stride},
+                                 state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
+                                 n_chunks, carry, out, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -7,6 +7,16 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+// Which keys a position sees, as one number that every attention kernel takes in its `window`
+// place: 0: all keys up to its own; n > 0: the last n (a sliding window); n < 0: those of its
+// own chunk of -n positions, chunks counted from position 0 of the sequence.  The first key seen
+// never moves back as the position grows, which is all the kernels' tile bounds rely on.
+__host__ __device__ __forceinline__ int kappai_first_key(int pos, int window) {
+  if (window > 0) return pos + 1 > window ? pos + 1 - window : 0;
+  if (window < 0) return pos < 0 ? 0 : pos - pos % (-window);
+  return 0;
+}
+
 struct kappai_score_mods {
   float softcap;
   const float* dist_bias;

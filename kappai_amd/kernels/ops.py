@@ -344,6 +344,16 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def tanh(x: torch.Tensor) -> torch.Tensor:
+    """``tanh`` of every element, stored as ``x`` is."""
+    _gpu("x", x, (F32, BF16))
+    out = torch.empty_like(x)
+    check(library("elementwise").kappai_unary(
+        _ptr(x), _ptr(out), _c_long(x.numel()), _c_int(0), _c_int(_is_bf16(x.dtype)), _stream()),
+        "tanh")
+    return out
+
+
 def cast(x: torch.Tensor, dtype) -> torch.Tensor:
     _gpu("x", x, (F32, BF16))
     if x.dtype == dtype:
@@ -859,12 +869,18 @@ class QkPrologue:
     store_kv: bool = True
 
 
+def keys_bound(max_position: int, window: int) -> int:
+    """An upper bound of the keys a row at ``max_position`` or before sees (``window``: 0 all,
+    n > 0 a sliding window of n, n < 0 chunks of -n positions; rounded as the kernels' tiles)."""
+    return min(max_position + 1, abs(window)) + 32 if window else max_position + 1
+
+
 def decode_form(n_heads: int, n_kv_heads: int, head_dim: int, max_position: int,
                 window: int = 0) -> str:
     """Which of the two decode kernels a step takes: with few keys ("decode-block") a block per
     (row, kv head) splits them over its waves and merges in LDS; else ("decode-split") the keys
     are split over blocks, whose partial results a second kernel merges."""
-    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    n_keys = keys_bound(max_position, window)
     lib = library("attention_mfma", HEAD_DIM=head_dim)
     block_waves = lib.kappai_attn_decode_block_waves(n_heads // n_kv_heads)
     return "decode-block" if block_waves and n_keys <= DECODE_BLOCK_MAX_KEYS else "decode-split"
@@ -886,9 +902,11 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                     kernel: str = "auto", prefill_variant: int = 0,
                     qk: Optional[QkPrologue] = None, lone_rows: Optional[torch.Tensor] = None,
                     max_lone_position: int = -1,
-                    mods: Optional[ScoreMods] = None) -> torch.Tensor:
+                    mods: Optional[ScoreMods] = None, chunk: int = 0) -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
-    (its own included; the last ``window`` of them when a window is set).  ``q`` is
+    (its own included; the last ``window`` of them when a window is set; with ``chunk`` those of
+    its own chunk of that many positions, chunks counted from position 0: the kernels take a
+    chunk as a negative window).  ``q`` is
     [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
 
     bfloat16 with a page size and head size that are multiples of 16 runs on the matrix
@@ -910,6 +928,10 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
 
     ``mods`` (``ScoreMods``): a cap on the scores, a bias by distance, a sink."""
     H, G, d = n_heads, n_kv_heads, head_dim
+    _need(not (window and chunk) and (window or 0) >= 0 and chunk >= 0,
+          "paged_attention: a sliding window or chunks, not both")
+    if chunk:
+        window = -int(chunk)
     if mods is not None and not mods.active():
         mods = None
     mods_c = mods.c_struct(H) if mods is not None else None
@@ -997,7 +1019,7 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                           f"{max_position} of heads of {d}")
         qk_args = (_ptr(qk.q_norm_w), _ptr(qk.k_norm_w), _c_float(qk.eps), _ptr(qk.cos),
                    _ptr(qk.sin), _c_int(1 if qk.store_kv else 0))
-    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    n_keys = keys_bound(max_position, window)
     block_waves = lib.kappai_attn_decode_block_waves(H // G)
     if kernel == "decode":
         kernel = "decode-split" if qk is not None else decode_form(H, G, d, max_position, window)
@@ -1031,7 +1053,7 @@ def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_table
     """The decode kernel that splits a row's keys over blocks, and its merge, for all rows or
     (``row_ids``) some of them."""
     T = q.shape[0] if row_ids is None else row_ids.shape[0]
-    n_keys = min(max_position + 1, window) + 32 if window else max_position + 1
+    n_keys = keys_bound(max_position, window)
     # one wave keeps the loads of `kpw` keys in flight; splits are whole numbers of that, and
     # at most DECODE_MAX_SPLITS of them are merged
     kpw = lib.kappai_attn_keys_per_wave()
@@ -1390,6 +1412,53 @@ def mingru_scan(proj: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor
     return out
 
 
+def gated_unit_scan(gates: torch.Tensor, gate_bias: torch.Tensor, u: torch.Tensor,
+                    y: torch.Tensor, softplus_lam: torch.Tensor,
+                    rate: float, state: torch.Tensor, seg_start: torch.Tensor,
+                    seg_pos0: torch.Tensor, seg_slot: torch.Tensor,
+                    chunks: Optional[torch.Tensor] = None,
+                    seg_chunk0: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The real-gated linear unit per channel: ``a = exp(-rate * sigmoid(g_r) * softplus_lam)``,
+    ``S = a S + sqrt(1 - a^2) * sigmoid(g_i) * u``, output ``S * gelu_tanh(y)``.  ``gates``
+    [T, 2W] float32 = (g_r | g_i) before the sigmoid and without ``gate_bias`` [2W], ``u`` [T, W], ``y`` [T, >= W] (a view with a
+    row stride) as a product stored them, ``softplus_lam`` [W] float32, ``state`` [slots, W]
+    float32.  ``chunks`` / ``seg_chunk0`` as for ``mingru_scan``.  Returns [T, W] as ``u`` is
+    stored."""
+    _gpu("gates", gates, F32)
+    _gpu("gate_bias", gate_bias, F32)
+    _gpu("u", u, (F32, BF16))
+    _gpu("y", y, u.dtype, contiguous=False)
+    _gpu("softplus_lam", softplus_lam, F32)
+    _gpu("state", state, F32)
+    T, W = u.shape
+    _need(tuple(gates.shape) == (T, 2 * W) and gate_bias.shape == (2 * W,) and y.dim() == 2 and y.shape[0] == T
+          and y.shape[1] >= W and y.stride(1) == 1 and softplus_lam.shape == (W,)
+          and state.dim() == 2 and state.shape[1] == W,
+          lambda: f"gated_unit_scan: gates {tuple(gates.shape)}, u {tuple(u.shape)}, y "
+                  f"{tuple(y.shape)}, state {tuple(state.shape)}")
+    for name, t in (("seg_start", seg_start), ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    _need(seg_start.shape[0] == S + 1 and seg_pos0.shape[0] == S,
+          "gated_unit_scan: segment tables do not fit")
+    out = torch.empty((T, W), dtype=u.dtype, device=u.device)
+    n_chunks, carry = 0, None
+    if chunks is not None:
+        _gpu("chunks", chunks, I32)
+        _gpu("seg_chunk0", seg_chunk0, I32)
+        _need(chunks.dim() == 2 and chunks.shape[1] == 3 and seg_chunk0.shape[0] == S + 1,
+              "gated_unit_scan: chunk tables do not fit")
+        n_chunks = chunks.shape[0]
+        carry = torch.empty((n_chunks, 3, W), dtype=F32, device=u.device)
+    check(library("mingru").kappai_gated_unit_scan(
+        _ptr(gates), _ptr(gate_bias), _ptr(u), _ptr(y), _c_int(y.stride(0)), _ptr(softplus_lam),
+        _c_float(rate),
+        _c_int(_is_bf16(u.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot),
+        _c_int(T), _c_int(S), _c_int(W), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks),
+        _ptr(carry), _ptr(out), _stream()), "gated_unit_scan")
+    return out
+
+
 # ---------------------------------------------------------------------------------------
 # differential attention: the two maps of a head as heads of the paged attention kernels
 # ---------------------------------------------------------------------------------------
@@ -1648,6 +1717,49 @@ def output_norm_add(resid: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, 
     return rows
 
 
+def pair_norm_sum(a: torch.Tensor, b: torch.Tensor, scale_a: float = 1.0, scale_b: float = 1.0,
+                  weight_a: Optional[torch.Tensor] = None,
+                  weight_b: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+    """``scale_a * n_a(a) + scale_b * n_b(b)`` in float32, ``n(y) = y / sqrt(mean(y^2) + eps) * w``
+    where a weight [D] is given and ``y`` itself where not.  ``a``, ``b`` [T, D] in one dtype
+    (float32 or bfloat16).  Returns float32 [T, D]."""
+    _gpu("a", a, (F32, BF16))
+    _gpu("b", b, a.dtype)
+    _need(a.dim() == 2 and a.shape == b.shape, lambda: f"pair_norm_sum: {tuple(a.shape)} and "
+                                                       f"{tuple(b.shape)}")
+    T, D = a.shape
+    for name, w in (("weight_a", weight_a), ("weight_b", weight_b)):
+        if w is not None:
+            _gpu(name, w, F32)
+            _need(w.shape == (D,), lambda: f"pair_norm_sum: {name} {tuple(w.shape)}")
+    out = torch.empty((T, D), dtype=F32, device=a.device)
+    check(library("elementwise").kappai_pair_norm_sum(
+        _ptr(a), _c_float(scale_a), _ptr(weight_a), _ptr(b), _c_float(scale_b), _ptr(weight_b),
+        _c_float(eps), _c_int(T), _c_int(D), _ptr(out), _c_int(_is_bf16(a.dtype)), _stream()),
+        "pair_norm_sum")
+    return out
+
+
+def stream_enter(resid: torch.Tensor, delta: Optional[torch.Tensor],
+                 again: Optional[torch.Tensor], row: Optional[torch.Tensor]) -> None:
+    """``resid += delta`` (a pending update [T, D], float32 or bfloat16, or None), ``+= again``
+    (float32 [T, D] or None), ``+= row`` (float32 [D] or None), in this order, in place."""
+    _gpu("resid", resid, F32)
+    T, D = resid.shape
+    if delta is not None:
+        _gpu("delta", delta, (F32, BF16))
+        _need(tuple(delta.shape) == (T, D), lambda: f"stream_enter: delta {tuple(delta.shape)}")
+    if again is not None:
+        _gpu("again", again, F32)
+        _need(tuple(again.shape) == (T, D), lambda: f"stream_enter: again {tuple(again.shape)}")
+    if row is not None:
+        _gpu("row", row, F32)
+        _need(tuple(row.shape) == (D,), lambda: f"stream_enter: row {tuple(row.shape)}")
+    check(library("elementwise").kappai_stream_enter(
+        _ptr(resid), _ptr(delta), _c_int(_is_bf16(delta.dtype) if delta is not None else 0),
+        _ptr(again), _ptr(row), _c_int(T), _c_int(D), _stream()), "stream_enter")
+
+
 # ---------------------------------------------------------------------------------------
 # attention layers whose queries, keys and values are not the plain grouped-query form
 # ---------------------------------------------------------------------------------------
@@ -1692,6 +1804,51 @@ def projection_norm_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim
         _ptr(block_tables if store_kv else None), _c_int(max_blocks), _c_int(T), _c_int(H),
         _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size), _ptr(q),
         _c_int(_is_bf16(proj.dtype)), _stream()), "projection_norm_store")
+    return q
+
+
+def rotate_widen_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, vdim: int,
+                       head_size: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                       rot_dims: int, rot_mode: int, values_are_keys: bool,
+                       k_pool: torch.Tensor, v_pool: torch.Tensor, row_pos: torch.Tensor,
+                       row_seg: torch.Tensor, block_tables: torch.Tensor,
+                       page_size: int) -> torch.Tensor:
+    """From ``proj`` [T, H dim + G dim (+ G vdim)]: the first ``rot_dims`` places of every q and
+    k head turn by the row's position (``cos`` / ``sin`` [positions, rot_dims / 2] float32, with
+    whatever factor the encoding puts on them; ``rot_mode`` as ``qk_norm_rope_store``).  Returns
+    queries [T, H head_size] (zeros behind ``dim``); keys and values go to pools made for G kv
+    heads of ``head_size``.  ``values_are_keys``: there are no value columns; a kv head's value
+    is its key as projected, before the rotation."""
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    _gpu("proj", proj, (F32, BF16), contiguous=False)
+    T = proj.shape[0]
+    need = H * d + G * d + (0 if values_are_keys else G * dv)
+    _need(proj.dim() == 2 and proj.shape[1] >= need and proj.stride(1) == 1,
+          lambda: f"rotate_widen_store: proj {tuple(proj.shape)} holds fewer than {need} columns")
+    _need(H % G == 0 and d <= D and dv <= D and (not values_are_keys or dv == d),
+          lambda: f"rotate_widen_store: {H} heads over {G}, sizes {d} and {dv} in heads of {D}")
+    if rot_mode != ROT_NONE and rot_dims:
+        _gpu("cos", cos, F32)
+        _gpu("sin", sin, F32)
+        _need(rot_dims % 2 == 0 and rot_dims <= d and cos.shape == sin.shape and cos.dim() == 2
+              and cos.shape[1] == rot_dims // 2,
+              lambda: f"rotate_widen_store: tables {tuple(cos.shape)} for {rot_dims} places of {d}")
+    else:
+        rot_dims, rot_mode, cos, sin = 0, ROT_NONE, None, None
+    _gpu("k_pool", k_pool, proj.dtype)
+    _gpu("v_pool", v_pool, proj.dtype)
+    _check_pools(k_pool, v_pool, G, page_size, D)
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("block_tables", block_tables)):
+        _gpu(name, t, I32)
+    _need(row_pos.shape[0] == T and row_seg.shape[0] == T and block_tables.dim() == 2,
+          "rotate_widen_store: row tables do not fit the batch")
+    q = torch.empty((T, H * D), dtype=proj.dtype, device=proj.device)
+    check(library("attn_prep").kappai_rotate_widen_store(
+        _ptr(proj), _c_int(proj.stride(0)), _ptr(cos), _ptr(sin), _c_int(rot_dims),
+        _c_int(rot_mode), _c_int(1 if values_are_keys else 0), _ptr(k_pool), _ptr(v_pool),
+        _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
+        _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size),
+        _ptr(q), _c_int(_is_bf16(proj.dtype)), _stream()), "rotate_widen_store")
     return q
 
 
@@ -1740,10 +1897,10 @@ def latent_store(q: torch.Tensor, kv: torch.Tensor, n_heads: int, dim: int, rot_
 
 
 def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor,
-                    out: Optional[torch.Tensor] = None, out_head_stride: Optional[int] = None
-                    ) -> torch.Tensor:
+                    out: Optional[torch.Tensor] = None, out_head_stride: Optional[int] = None,
+                    out_dtype=None) -> torch.Tensor:
     """``y[t, h, :] = weight[h] @ x[t, h, :]`` with ``weight`` [H, n_out, n_in] in the dtype of
-    ``x``.  Head h of row t starts at ``x[t, h * x_head_stride]`` and is written at
+    ``x``.  ``out_dtype`` float32 keeps the sums as they are (else they are stored as ``x`` is).  Head h of row t starts at ``x[t, h * x_head_stride]`` and is written at
     ``out[t, h * out_head_stride]`` (``out`` None: a new [T, H n_out])."""
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, x.dtype)
@@ -1753,17 +1910,20 @@ def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor,
     _need(x.dim() == 2 and x.stride(1) == 1 and (H - 1) * x_head_stride + n_in <= x.shape[1],
           lambda: f"headwise_linear: x {tuple(x.shape)} for {H} heads of {n_in} every "
                   f"{x_head_stride}")
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    _need(out_dtype in (x.dtype, F32), "headwise_linear: results as x is stored, or float32")
     if out is None:
-        out = torch.empty((T, H * n_out), dtype=x.dtype, device=x.device)
+        out = torch.empty((T, H * n_out), dtype=out_dtype, device=x.device)
         out_head_stride = n_out
-    _gpu("out", out, x.dtype, contiguous=False)
+    _gpu("out", out, out_dtype, contiguous=False)
     _need(out.dim() == 2 and out.shape[0] == T and out.stride(1) == 1
           and (H - 1) * out_head_stride + n_out <= out.shape[1],
           lambda: f"headwise_linear: out {tuple(out.shape)}")
     check(library("attn_prep").kappai_headwise_linear(
         _ptr(x), _c_int(x.stride(0)), _c_int(x_head_stride), _ptr(weight), _c_int(H),
         _c_int(n_out), _c_int(n_in), _ptr(out), _c_int(out.stride(0)), _c_int(out_head_stride),
-        _c_int(T), _c_int(_is_bf16(x.dtype)), _stream()), "headwise_linear")
+        _c_int(T), _c_int(_is_bf16(x.dtype)), _c_int(1 if out_dtype == F32 else 0), _stream()),
+        "headwise_linear")
     return out
 
 
@@ -1775,8 +1935,10 @@ CONV_SILU_MAX_TAPS = 17
 
 def conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos: torch.Tensor,
               row_seg: torch.Tensor, seg_start: torch.Tensor, seg_pos0: torch.Tensor,
-              seg_slot: torch.Tensor) -> torch.Tensor:
-    """``silu(conv(x))`` per channel: ``conv(x)[t] = sum_j taps[:, j] x[t - n + 1 + j]``, zeros
+              seg_slot: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              activation: bool = True) -> torch.Tensor:
+    """``silu(conv(x) + bias)`` per channel (``activation`` False: no SiLU; ``bias`` [C] float32
+    or None): ``conv(x)[t] = sum_j taps[:, j] x[t - n + 1 + j]``, zeros
     before position 0.  ``x`` [T, >= C] (a view with a row stride), ``taps`` [C, n] float32,
     ``state`` [slots, n - 1, C] float32: the request's last inputs, read for rows before the
     step's portion and brought up to date.  Returns [T, C] in the dtype of ``x``."""
@@ -1793,30 +1955,73 @@ def conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos:
                     ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
         _gpu(name, t, I32)
     S = seg_slot.shape[0]
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (C,), lambda: f"conv_silu: bias {tuple(bias.shape)} for {C} channels")
     out = torch.empty((T, C), dtype=x.dtype, device=x.device)
     check(library("linear_attention").kappai_conv_silu(
         _ptr(x), _c_int(x.stride(0)), _ptr(taps), _c_int(n), _ptr(state), _ptr(row_pos),
         _ptr(row_seg), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(S),
-        _c_int(C), _ptr(out), _c_int(_is_bf16(x.dtype)), _stream()), "conv_silu")
+        _c_int(C), _ptr(bias), _c_int(1 if activation else 0), _ptr(out),
+        _c_int(_is_bf16(x.dtype)), _stream()), "conv_silu")
+    return out
+
+
+def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor,
+                    row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,
+                    seg_slot: torch.Tensor) -> torch.Tensor:
+    """``out[m] = h + (h' - h) * mu[m]`` with ``h'`` the row of the token before (zeros at position
+    0): ``h`` [T, W], ``mu`` [n, W] float32, ``state`` [slots, W] float32 (the request's last row,
+    read for a segment's first row and brought up to date).  Returns [n, T, W] as ``h`` is stored."""
+    _gpu("h", h, (F32, BF16), contiguous=False)
+    _gpu("mu", mu, F32)
+    _gpu("state", state, F32)
+    T, W = h.shape
+    _need(h.stride(1) == 1 and mu.dim() == 2 and mu.shape[1] == W
+          and tuple(state.shape[1:]) == (W,),
+          lambda: f"token_shift_mix: h {tuple(h.shape)}, mu {tuple(mu.shape)}, state "
+                  f"{tuple(state.shape)}")
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("seg_start", seg_start),
+                    ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    out = torch.empty((mu.shape[0], T, W), dtype=h.dtype, device=h.device)
+    check(library("linear_attention").kappai_token_shift_mix(
+        _ptr(h), _c_int(h.stride(0)), _ptr(mu), _c_int(mu.shape[0]), _ptr(state), _ptr(row_pos),
+        _ptr(row_seg), _ptr(seg_start), _ptr(seg_slot), _c_int(T), _c_int(S), _c_int(W),
+        _ptr(out), _c_int(_is_bf16(h.dtype)), _stream()), "token_shift_mix")
     return out
 
 
 SCAN_FORMS = {"auto": 0, "wave": 1, "block": 2}
 
 
-def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
+DECAY_KINDS = {"softplus": 0, "double_exp": 1, "fixed": 2}
+
+
+def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                            z: Optional[torch.Tensor],
                             n_heads: int, n_qk_heads: int, dim: int, vdim: int,
-                            rate: torch.Tensor, z_bias: Optional[torch.Tensor], z_sign: float,
+                            rate: Optional[torch.Tensor], z_bias: Optional[torch.Tensor],
+                            z_sign: float,
                             q_scale: float, state: torch.Tensor, seg_start: torch.Tensor,
                             seg_pos0: torch.Tensor, seg_slot: torch.Tensor,
                             beta: Optional[torch.Tensor] = None, unit_qk: bool = False,
-                            unit_eps: float = 1e-6, form: str = "auto") -> torch.Tensor:
+                            unit_eps: float = 1e-6, form: str = "auto",
+                            decay: str = "softplus", bonus: Optional[torch.Tensor] = None,
+                            silu_inputs: bool = False) -> torch.Tensor:
     """A state ``S`` [dim, vdim] per head, float32, kept column by column in ``state``
     [slots, H, vdim, dim] (a segment that starts at position 0 starts from zero).  Per token, with the decay per key channel
     ``a = exp(-rate[h] * softplus(z_sign * (z + z_bias)))``:
     without ``beta``   ``S <- diag(a) S + k v^T``, ``o = S^T q``;
     with ``beta``      ``S <- diag(a) S``, ``u = sigmoid(beta) (v - S^T k)``, ``S <- S + k u^T``,
-                       ``o = S^T q`` (the delta rule; the read-out sees the token's own write).
+                       ``o = S^T q`` (the delta rule; the read-out sees the token's own write);
+    with ``bonus``     ``o = (S + diag(bonus[h]) k v^T)^T q``, then ``S <- diag(a) S + k v^T`` (the
+                       read-out sees the state before the token, and the token itself weighed by
+                       ``bonus`` [H, dim] float32).
+    ``decay`` = "double_exp": ``a = exp(-exp(z + z_bias))``; "fixed": ``a = rate[h]`` for every
+    token and channel (``z`` None).  ``silu_inputs``: q, k and v pass SiLU first (rounded as they
+    are stored).
     ``q``, ``k`` [T, Hk dim] (head h reads q/k head ``h // (H / Hk)``; ``unit_qk``: each head's
     vector divided by ``sqrt(sum x^2 + unit_eps)`` first), q times ``q_scale``; ``v`` [T, H vdim];
     ``z`` [T, H dim]; ``beta`` [T, H]; all views with a row stride.  Everything between the
@@ -1826,8 +2031,15 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
     token from global memory, or a block of waves that takes the tokens in chunks through LDS."""
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     _need(form in SCAN_FORMS, lambda: f"matrix_state_recurrence: form {form!r}")
+    _need(decay in DECAY_KINDS and (z is None) == (decay == "fixed")
+          and (rate is not None or decay == "double_exp"),
+          lambda: f"matrix_state_recurrence: decay {decay!r} with z {'given' if z is not None else 'missing'}")
+    _need(beta is None or bonus is None, "matrix_state_recurrence: the delta rule or a bonus")
+    _need(not (silu_inputs and unit_qk), "matrix_state_recurrence: SiLU or unit vectors")
     T = q.shape[0]
     for name, t, cols in (("q", q, Hk * d), ("k", k, Hk * d), ("v", v, H * dv), ("z", z, H * d)):
+        if t is None:
+            continue
         _gpu(name, t, q.dtype, contiguous=False)
         _need(t.dim() == 2 and t.shape[0] == T and t.shape[1] >= cols and t.stride(1) == 1,
               lambda: f"matrix_state_recurrence: {name} {tuple(t.shape)}, expected [T, {cols}]")
@@ -1836,8 +2048,13 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
         _gpu("beta", beta, q.dtype, contiguous=False)
         _need(beta.dim() == 2 and beta.shape[0] == T and beta.shape[1] >= H
               and (beta.stride(1) == 1 or H == 1), "matrix_state_recurrence: beta must be [T, H]")
-    _gpu("rate", rate, F32)
-    _need(rate.shape == (H,), "matrix_state_recurrence: one rate a head")
+    if rate is not None:
+        _gpu("rate", rate, F32)
+        _need(rate.shape == (H,), "matrix_state_recurrence: one rate a head")
+    if bonus is not None:
+        _gpu("bonus", bonus, F32)
+        _need(tuple(bonus.shape) == (H, d) and H == Hk,
+              lambda: f"matrix_state_recurrence: bonus {tuple(bonus.shape)} for {H} heads of {d}")
     if z_bias is not None:
         _gpu("z_bias", z_bias, F32)
         _need(z_bias.shape == (H * d,), "matrix_state_recurrence: z_bias must be [H dim]")
@@ -1852,19 +2069,28 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
     kf = torch.empty((T, Hk * d), dtype=F32, device=dev)
     af = torch.empty((T, H * d), dtype=F32, device=dev)
     bf = torch.empty((T, H), dtype=F32, device=dev) if beta is not None else None
+    vf = torch.empty((T, H * dv), dtype=F32, device=dev) if silu_inputs else None
     lib = library("linear_attention")
     check(lib.kappai_recurrence_prep(
-        _ptr(q), _c_int(q.stride(0)), _ptr(k), _c_int(k.stride(0)), _ptr(z), _c_int(z.stride(0)),
+        _ptr(q), _c_int(q.stride(0)), _ptr(k), _c_int(k.stride(0)), _ptr(z),
+        _c_int(z.stride(0) if z is not None else 0),
         _ptr(z_bias), _ptr(rate), _c_float(z_sign), _ptr(beta),
         _c_int(beta.stride(0) if beta is not None else 0), _c_int(T), _c_int(H), _c_int(Hk),
-        _c_int(d), _c_int(1 if unit_qk else 0), _c_float(unit_eps), _c_float(q_scale), _ptr(qf),
-        _ptr(kf), _ptr(af), _ptr(bf), _c_int(_is_bf16(q.dtype)), _stream()), "recurrence_prep")
+        _c_int(d), _c_int(1 if unit_qk else 0), _c_float(unit_eps), _c_float(q_scale),
+        _c_int(1 if silu_inputs else 0), _c_int(DECAY_KINDS[decay]),
+        _ptr(v if silu_inputs else None), _c_int(v.stride(0)), _c_int(dv), _ptr(qf),
+        _ptr(kf), _ptr(af), _ptr(bf), _ptr(vf), _c_int(_is_bf16(q.dtype)), _stream()),
+        "recurrence_prep")
     out = torch.empty((T, H * dv), dtype=F32, device=dev)
+    values = vf if silu_inputs else v
+    mode = 1 if beta is not None else 2 if bonus is not None else 0
     check(lib.kappai_matrix_state_scan(
-        _ptr(qf), _ptr(kf), _ptr(af), _ptr(bf), _ptr(v), _c_int(v.stride(0)),
-        _c_int(_is_bf16(v.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot),
+        _ptr(qf), _ptr(kf), _ptr(af), _ptr(bonus if bonus is not None else bf), _ptr(values),
+        _c_int(values.stride(0)),
+        _c_int(_is_bf16(values.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0),
+        _ptr(seg_slot),
         _c_int(T), _c_int(S), _c_int(H), _c_int(Hk), _c_int(d), _c_int(dv),
-        _c_int(1 if beta is not None else 0), _c_int(SCAN_FORMS[form]), _ptr(out), _stream()),
+        _c_int(mode), _c_int(SCAN_FORMS[form]), _ptr(out), _stream()),
         "matrix_state_scan")
     return out
 
@@ -1874,20 +2100,22 @@ GATE_SILU, GATE_SIGMOID = 0, 1
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor,
                    gate_kind: int, n_heads: int, vdim: int, out_dtype) -> torch.Tensor:
-    """Per head ``o / sqrt(mean(o^2) + eps) * weight`` (``weight`` [vdim], shared by the heads)
-    times ``silu(gate)`` or ``sigmoid(gate)``: ``o`` [T, H vdim] float32, ``gate`` [T, >= H vdim]
+    """Per head ``o / sqrt(mean(o^2) + eps) * weight`` (``weight`` [vdim], shared by the heads, or
+    [H, vdim], one a head) times ``silu(gate)`` or ``sigmoid(gate)``: ``o`` [T, H vdim] float32, ``gate`` [T, >= H vdim]
     in ``out_dtype`` (a view with a row stride).  Returns [T, H vdim] in ``out_dtype``."""
     H, dv = n_heads, vdim
     _gpu("o", o, F32)
     _gpu("weight", weight, F32)
     _gpu("gate", gate, out_dtype, contiguous=False)
     T = o.shape[0]
-    _need(tuple(o.shape) == (T, H * dv) and weight.shape == (dv,) and gate.dim() == 2
+    _need(tuple(o.shape) == (T, H * dv) and tuple(weight.shape) in ((dv,), (H, dv))
+          and gate.dim() == 2
           and gate.shape[0] == T and gate.shape[1] >= H * dv and gate.stride(1) == 1,
           lambda: f"head_norm_gate: o {tuple(o.shape)}, gate {tuple(gate.shape)}")
     out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
     check(library("linear_attention").kappai_head_norm_gate(
         _ptr(o), _ptr(weight), _c_float(eps), _ptr(gate), _c_int(gate.stride(0)),
-        _c_int(gate_kind), _c_int(T), _c_int(H), _c_int(dv), _ptr(out),
+        _c_int(gate_kind), _c_int(T), _c_int(H), _c_int(dv),
+        _c_int(dv if weight.dim() == 2 else 0), _ptr(out),
         _c_int(_is_bf16(out_dtype)), _stream()), "head_norm_gate")
     return out

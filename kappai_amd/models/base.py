@@ -5,6 +5,10 @@ block may be named more than once (then every call has a cache of its own), and 
 may read the cache that an earlier call wrote instead of owning one (``reads_cache_of``).
 The caches are numbered by the calls that own them; the cache manager groups them by
 what they need.
+
+A call may also name an entry (``enters``, an index into ``Model.entries``): a part that works on
+the stream itself right before the call's block (``parts.passes.PassEntry``: what a pass over a
+run of layers starts with).  It gets the stream and the embedded rows as they left the embedding.
 """
 from __future__ import annotations
 
@@ -24,6 +28,7 @@ from ..weights.spec import TensorSpec
 class LayerCall:
     layer: int                            # index into Model.layers
     reads_cache_of: Optional[int] = None  # index into the schedule of the call whose cache is read
+    enters: Optional[int] = None          # index into Model.entries: runs on the stream before
 
 
 class Model:
@@ -31,7 +36,7 @@ class Model:
                  layers: Sequence[Block], final_norm: Norm, head: OutputHead,
                  schedule: Optional[Sequence[LayerCall]] = None,
                  embedding_position: Optional[PositionEncoding] = None,
-                 embedding_norm: Optional[Norm] = None):
+                 embedding_norm: Optional[Norm] = None, entries: Sequence = ()):
         """``embedding_norm``: a norm that the embedded rows pass before the first layer (one with
         ``norm_output``); the stream then starts as the normalised rows."""
         self.config, self.dtype = config, dtype
@@ -39,6 +44,7 @@ class Model:
         self.final_norm, self.head = final_norm, head
         self.embedding_position = embedding_position
         self.embedding_norm = embedding_norm
+        self.entries = list(entries)
         # names a checkpoint may hold although this model reads none of them (a builder fills it)
         self.unused_tensor_names: List[str] = []
         self.schedule: List[LayerCall] = list(schedule) if schedule is not None else [
@@ -51,6 +57,9 @@ class Model:
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"schedule[{ci}] names layer {call.layer}; there are "
                                  f"{len(self.layers)}")
+            if call.enters is not None and not 0 <= call.enters < len(self.entries):
+                raise ValueError(f"schedule[{ci}] names entry {call.enters}; there are "
+                                 f"{len(self.entries)}")
             src = call.reads_cache_of
             if src is not None:
                 if not 0 <= src < ci:
@@ -76,7 +85,7 @@ class Model:
 
     # -- weights ---------------------------------------------------------------------------
     def _parts(self):
-        parts = [self.embedding, *self.layers, self.final_norm, self.head]
+        parts = [self.embedding, *self.layers, *self.entries, self.final_norm, self.head]
         if self.embedding_position is not None:
             parts.append(self.embedding_position)
         if self.embedding_norm is not None:
@@ -143,6 +152,8 @@ class Model:
         calls = []
         if self.embedding_norm is not None:
             return None            # the walk from C knows no norm between embedding and layers
+        if any(call.enters is not None for call in self.schedule):
+            return None            # nor parts that work on the stream between two blocks
         for ci, call in enumerate(self.schedule):
             block = self.layers[call.layer]
             if not defined_together(block, "forward", "c_call"):
@@ -169,14 +180,21 @@ class Model:
             narrow = self.dtype != torch.float32
             h.rows = self.embedding_norm.norm_output(x, x, add=False,
                                                      rows_dtype=self.dtype if narrow else None)
+        embedded = None
+        if any(getattr(e, "reads_embedded", False) for e in self.entries):
+            embedded = x.clone()       # the blocks change the stream in place
         for ci, call in enumerate(self.schedule):
             block = self.layers[call.layer]
             view = None
             if block.cache_spec() is not None:
                 view = cache.view(self.cache_id(ci))
             shared = call.reads_cache_of is not None
+            if call.enters is not None:
+                h = self.entries[call.enters].forward(h, embedded, batch)
             if getattr(block, "takes_next_block", False):
-                if ci + 1 < len(self.schedule):
+                if ci + 1 < len(self.schedule) and self.schedule[ci + 1].enters is not None:
+                    nxt = None         # the stream changes before the next block's first norm
+                elif ci + 1 < len(self.schedule):
                     nxt = self.layers[self.schedule[ci + 1].layer]
                 else:
                     # after the last call comes the final norm, whose rows the head takes; a

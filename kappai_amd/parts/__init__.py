@@ -5,15 +5,18 @@ from .block import ConvInputBlock, OutputNormBlock, PreNormBlock
 from .diff_attention import DifferentialAttention
 from .embedding import OutputHead, TokenEmbedding
 from .feed_forward import SwiGLU
+from .gated_unit import RealGatedUnit
 from .group_norm import GroupRMSNorm
 from .input_conv import ShortInputConv
 from .latent_attention import LatentAttention
 from .linear import Linear
-from .linear_attention import GatedDeltaRule, GatedLinearAttention
+from .linear_attention import (BonusTimeMixing, FixedDecayAttention, GatedDeltaRule,
+                               GatedLinearAttention)
 from .mingru import MinGRU
 from .moe import MixtureOfExperts
 from .norm import RMSNorm
 from .parallel import ParallelMixer
+from .passes import PassEntry
 from .positions import LearnedPositions
 from .rotary import RotaryEncoding, Rotation
 from .scored_attention import ScoredAttention
@@ -26,4 +29,5 @@ __all__ = ["GroupedQueryAttention", "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS"
            "GatedShortConv", "ConvInputBlock", "DifferentialAttention", "GroupRMSNorm",
            "ShortInputConv", "MinGRU", "MixtureOfExperts", "LearnedPositions", "OutputNormBlock",
            "LatentAttention", "GatedDeltaRule", "GatedLinearAttention", "ParallelMixer",
-           "ScoredAttention"]
+           "ScoredAttention", "RealGatedUnit", "BonusTimeMixing", "FixedDecayAttention",
+           "PassEntry"]

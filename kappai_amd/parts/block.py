@@ -26,14 +26,19 @@ def _takes_defer(norm) -> bool:
 class PreNormBlock(Block):
     """``x += mixer(norm(x)); x += feed_forward(norm(x))`` (kappai: src/models/lfm.c:7-53 with
     the tail src/recipe/builders.c:378-388).  Each residual sum is made inside the norm
-    that follows it."""
+    that follows it.  ``feed_forward`` (with its norm) may be None: the layer is then its mixer
+    alone."""
 
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, feed_forward: FeedForward):
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm = None,
+                 feed_forward: FeedForward = None):
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.mixer_norm, self.mixer = mixer_norm, mixer
         self.ffn_norm, self.feed_forward = ffn_norm, feed_forward
 
     def _parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+                     if p is not None)
 
     @property
     def capturable(self) -> bool:
@@ -41,7 +46,12 @@ class PreNormBlock(Block):
 
     @property
     def step_tables(self):
-        return [t for t in (p.step_tables for p in self._parts()) if t is not None]
+        out = []
+        for p in self._parts():
+            asked = p.step_tables
+            if asked is not None:
+                out += list(asked) if isinstance(asked, (list, tuple)) else [asked]
+        return out
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self._parts() for s in p.tensor_specs()]
@@ -63,6 +73,10 @@ class PreNormBlock(Block):
         # itself and hand the next product its rows without a norm kernel in between
         resid = h.resid
         x = self._normed(self.mixer_norm, resid, h.delta, self.mixer)
+        if self.feed_forward is None:
+            # (no product of this layer folds anything in: the mixer's result is the update)
+            mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
+            return Hidden(self._resid_after(x, resid), mixed)
         into = self._into(self.mixer, resid, self.ffn_norm, self.feed_forward)
         if into is not None:
             mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache, into=into)
@@ -106,6 +120,8 @@ class PreNormBlock(Block):
         own descriptions side by side, or None when one of them has none.  A part whose class
         changed ``forward`` (or a norm's ``add_norm``) without giving a description of its own
         counts as having none."""
+        if self.feed_forward is None:
+            return None            # the runner on the C side knows the four-part layer only
         for part, method, c_method in ((self.mixer_norm, "add_norm", "c_norm"),
                                        (self.mixer, "forward", "c_part"),
                                        (self.ffn_norm, "add_norm", "c_norm"),

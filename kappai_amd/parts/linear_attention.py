@@ -14,6 +14,18 @@ write); each head's ``o`` divided by its root mean square, times a weight shared
 times ``sigmoid(W_g2 (W_g1 h))``, then ``W_o``.  The convolutions' last ``taps - 1`` inputs are
 state as well.
 
+``FixedDecayAttention``: ``q = silu(W_q h)``, ``k = silu(W_k h)``, ``v = silu(W_v h)``; one fixed
+decay a head, ``S <- decay[h] S + k v^T``, ``o = S^T q`` with no other scale; the heads side by
+side are RMS-normed TOGETHER with a weight [heads * vdim], times ``sigmoid(W_g h)``, then ``W_o``.
+
+``BonusTimeMixing``: with ``h'`` the token before (zeros at position 0), each of r, k, v, g, w
+reads its own mix ``h + (h' - h) * mu_s``; ``r, k, v = W_r, W_k, W_v`` of their mixes, the gate
+``silu(W_g mix_g)``, a decay per head and key channel ``w = exp(-exp(W_w2 tanh(W_w1 mix_w) +
+w0))``; per head ``o = (S + diag(u) k v^T)^T r`` (the bonus ``u`` [heads, dim] weighs the token
+itself, which the state does not hold yet), then ``S <- diag(w) S + k v^T``; each head's ``o``
+divided by its root mean square, times a weight [heads * dim] and the gate, then ``W_o``.  The
+last row of ``h`` is state as well.
+
 Projections, convolutions and their activations are stored in the compute dtype; decays,
 softplus, exponentials, step sizes, unit vectors, the state and the per-head norm are float32.
 """
@@ -99,6 +111,140 @@ class GatedLinearAttention(Mixer):
 
 
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+
+
+class FixedDecayAttention(Mixer):
+    def __init__(self, prefix: str, width: int, num_heads: int, dim: int, vdim: int, decay,
+                 norm_eps: float, dtype: torch.dtype, names=None, weight_suffix: str = ".weight"):
+        n = {"q": "q", "k": "k", "v": "v", "g": "g", "norm": "norm", "o": "o"}
+        n.update(names or {})
+        decay = [float(a) for a in decay]
+        if len(decay) != num_heads:
+            raise ValueError(f"{prefix}: {len(decay)} decays for {num_heads} heads")
+        if not all(0.0 <= a <= 1.0 for a in decay):
+            raise ValueError(f"{prefix}: a decay lies between 0 and 1, got {decay}")
+        self.prefix, self.width, self.dtype = prefix, width, dtype
+        self.H, self.d, self.dv, self.decay = num_heads, dim, vdim, decay
+        self.norm_eps = float(norm_eps)
+        H, d, dv = num_heads, dim, vdim
+        self.inputs = Linear([prefix + n[k] for k in ("q", "k", "v", "g")], width,
+                             [H * d, H * d, H * dv, H * dv], stage="matmul_in_proj",
+                             weight_suffix=weight_suffix)
+        self.out = Linear([prefix + n["o"]], H * dv, [width], stage="matmul_out_proj",
+                          weight_suffix=weight_suffix)
+        self._norm = prefix + n["norm"]
+        self.norm_w = self.rate = None
+
+    def cache_spec(self):
+        return FixedState((self.H, self.dv, self.d), "float32")
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return (self.inputs.tensor_specs() + self.out.tensor_specs()
+                + [TensorSpec(self._norm, (self.H * self.dv,), VECTOR, INIT_ONES)])
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.inputs.bind(tensors)
+        self.out.bind(tensors)
+        self.norm_w = tensors[self._norm].to(torch.float32).contiguous()
+        self.rate = torch.tensor(self.decay, dtype=torch.float64).to(torch.float32).to(
+            self.norm_w.device)
+
+    def forward(self, x, batch, cache, shared_cache: bool = False):
+        if shared_cache:
+            raise ValueError("a recurrent state cannot be read by another layer")
+        H, d, dv = self.H, self.d, self.dv
+        proj = self.inputs.forward(x)
+        o_k, o_v, o_g = H * d, 2 * H * d, 2 * H * d + H * dv
+        with profile.scope("scan"):
+            o = ops.matrix_state_recurrence(
+                proj, proj[:, o_k:], proj[:, o_v:], None, H, H, d, dv, self.rate, None, 1.0, 1.0,
+                cache.state, batch.seg_start, batch.seg_pos0, batch.seg_slot, decay="fixed",
+                silu_inputs=True)
+            # (all heads are normed together: one "head" of H * dv for the kernel)
+            y = ops.head_norm_gate(o, self.norm_w, self.norm_eps, proj[:, o_g:],
+                                   ops.GATE_SIGMOID, 1, H * dv, self.dtype)
+        return self.out.forward(y, partial_sums=True)
+
+    def weight_bytes(self) -> int:
+        return self.inputs.weight_bytes() + self.out.weight_bytes()
+
+
+register_part("mixer", "fixed_decay_attention", FixedDecayAttention)
+
+
+class BonusTimeMixing(Mixer):
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, prefix: str, width: int, num_heads: int, dim: int, decay_rank: int,
+                 norm_eps: float, dtype: torch.dtype, names=None, weight_suffix: str = ".weight"):
+        n = {"r": "r", "k": "k", "v": "v", "g": "g", "w1": "w1", "w2": "w2", "w0": "w0",
+             "u": "u", "mu": "mu.", "norm": "norm", "o": "o"}
+        n.update(names or {})
+        self.prefix, self.width, self.dtype = prefix, width, dtype
+        self.H, self.d, self.rank = num_heads, dim, int(decay_rank)
+        self.norm_eps = float(norm_eps)
+        H, d = num_heads, dim
+
+        def lin(key, n_in, n_out, stage="matmul_in_proj"):
+            return Linear([prefix + n[key]], n_in, [n_out], stage=stage,
+                          weight_suffix=weight_suffix)
+
+        self.r, self.k, self.v, self.g = (lin(s, width, H * d) for s in ("r", "k", "v", "g"))
+        self.w1, self.w2 = lin("w1", width, self.rank), lin("w2", self.rank, H * d)
+        self.out = lin("o", H * d, width, "matmul_out_proj")
+        self._mu = [prefix + n["mu"] + s for s in self.MIXES]
+        self._w0, self._u, self._norm = prefix + n["w0"], prefix + n["u"], prefix + n["norm"]
+        self.mu = self.w0 = self.bonus = self.norm_w = None
+
+    def _linears(self):
+        return (self.r, self.k, self.v, self.g, self.w1, self.w2, self.out)
+
+    def cache_spec(self):
+        return CacheBundle((("state", FixedState((self.H, self.d, self.d), "float32")),
+                            ("shift", FixedState((self.width,), "float32"))))
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [s for lin in self._linears() for s in lin.tensor_specs()]
+        specs += [TensorSpec(name, (self.width,), VECTOR, INIT_SMALL) for name in self._mu]
+        specs += [TensorSpec(self._w0, (self.H * self.d,), VECTOR, INIT_SMALL),
+                  TensorSpec(self._u, (self.H, self.d), VECTOR, INIT_SMALL),
+                  TensorSpec(self._norm, (self.H * self.d,), VECTOR, INIT_ONES)]
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for lin in self._linears():
+            lin.bind(tensors)
+        self.mu = torch.stack([tensors[name].to(torch.float32) for name in self._mu]).contiguous()
+        self.w0 = tensors[self._w0].to(torch.float32).contiguous()
+        self.bonus = tensors[self._u].to(torch.float32).contiguous()
+        self.norm_w = tensors[self._norm].to(torch.float32).reshape(self.H, self.d).contiguous()
+
+    def forward(self, x, batch, cache, shared_cache: bool = False):
+        if shared_cache:
+            raise ValueError("a recurrent state cannot be read by another layer")
+        H, d = self.H, self.d
+        with profile.scope("short_conv"):
+            mixes = ops.token_shift_mix(x, self.mu, cache.part("shift").state, batch.row_pos,
+                                        batch.row_seg, batch.seg_start, batch.seg_slot)
+        r, k, v, g = (lin.forward(mixes[i]) for i, lin in enumerate((self.r, self.k, self.v,
+                                                                     self.g)))
+        with profile.scope("ffn_act"):
+            low = ops.tanh(self.w1.forward(mixes[4]))
+        z = self.w2.forward(low)
+        with profile.scope("scan"):
+            o = ops.matrix_state_recurrence(
+                r, k, v, z, H, H, d, d, None, self.w0, 1.0, 1.0, cache.part("state").state,
+                batch.seg_start, batch.seg_pos0, batch.seg_slot, decay="double_exp",
+                bonus=self.bonus)
+            y = ops.head_norm_gate(o, self.norm_w, self.norm_eps, g, ops.GATE_SILU, H, d,
+                                   self.dtype)
+        return self.out.forward(y, partial_sums=True)
+
+    def weight_bytes(self) -> int:
+        return sum(lin.weight_bytes() for lin in self._linears())
+
+
+register_part("mixer", "bonus_time_mixing", BonusTimeMixing)
 
 
 class GatedDeltaRule(Mixer):

@@ -2,7 +2,13 @@
 ``left_scale * left(h) + right_scale * right(h)``.  The sum is left to whoever takes the result
 (``parts.base.WeightedTerms``: a norm on the sublayer's output adds the two in float32 while it
 normalises).  Each mixer keeps its own cache: the pair asks for a bundle with the members "left"
-and "right" (a member that is a bundle itself is taken apart: "left.<name>")."""
+and "right" (a member that is a bundle itself is taken apart: "left.<name>").
+
+``side_norms`` (two tensor names, with ``width`` and ``norm_eps``): each side's result is first
+RMS-normed over the model width with a plain weight of its own,
+``left_scale * n_l(left) + right_scale * n_r(right)``.  With side norms, or with ``summed``, the
+pair adds its two sides itself in float32 (one kernel) and returns that update, which any norm
+takes; an arrangement whose norm reads the mixer's input only needs this."""
 from __future__ import annotations
 
 from typing import Dict, List
@@ -12,15 +18,22 @@ import torch
 from ..cache.manager import BundleView
 from ..cache.specs import CacheBundle
 from ..kernels import ops
-from ..weights.spec import TensorSpec
+from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
 from .base import Mixer, WeightedTerms, register_part
 
 
 class ParallelMixer(Mixer):
     def __init__(self, left: Mixer, right: Mixer, left_scale: float = 1.0,
-                 right_scale: float = 1.0):
+                 right_scale: float = 1.0, summed: bool = False, side_norms=None,
+                 width: int = 0, norm_eps: float = 0.0):
         self.left, self.right = left, right
         self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self.side_norms = tuple(side_norms) if side_norms else None
+        if self.side_norms is not None and (len(self.side_norms) != 2 or width < 1):
+            raise ValueError("side norms are two tensor names, and need the model width")
+        self.summed = bool(summed) or self.side_norms is not None
+        self.width, self.norm_eps = int(width), float(norm_eps)
+        self.norm_w = (None, None)
 
     def _sides(self):
         return (("left", self.left), ("right", self.right))
@@ -58,11 +71,18 @@ class ParallelMixer(Mixer):
         return cache.part(side)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return self.left.tensor_specs() + self.right.tensor_specs()
+        specs = self.left.tensor_specs() + self.right.tensor_specs()
+        if self.side_norms is not None:
+            specs += [TensorSpec(name, (self.width,), VECTOR, INIT_ONES)
+                      for name in self.side_norms]
+        return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.left.bind(tensors)
         self.right.bind(tensors)
+        if self.side_norms is not None:
+            self.norm_w = tuple(tensors[name].to(torch.float32).contiguous()
+                                for name in self.side_norms)
 
     def forward(self, x, batch, cache, shared_cache: bool = False):
         if shared_cache:
@@ -75,10 +95,14 @@ class ParallelMixer(Mixer):
             out.append(y)
         if out[0].dtype != out[1].dtype:
             out = [y if y.dtype == torch.float32 else ops.cast(y, torch.float32) for y in out]
+        if self.summed:
+            return ops.pair_norm_sum(out[0], out[1], self.left_scale, self.right_scale,
+                                     self.norm_w[0], self.norm_w[1], self.norm_eps)
         return WeightedTerms(out[0], self.left_scale, out[1], self.right_scale)
 
     def weight_bytes(self) -> int:
-        return self.left.weight_bytes() + self.right.weight_bytes()
+        n = self.left.weight_bytes() + self.right.weight_bytes()
+        return n + (8 * self.width if self.side_norms is not None else 0)
 
 
 register_part("mixer", "parallel", ParallelMixer)

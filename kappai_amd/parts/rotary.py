@@ -5,11 +5,21 @@ precision and stored as float32, as kappai does (src/compute.c:22-56).  ``pairin
 "half" for rotate-half pairs (j, j + rot/2) (src/backend/cpu/quants.h:395-409) or
 "interleaved" for (2j, 2j+1) (src/backend/cpu/quants.h:411-438); ``rot_dim`` may be less
 than the head size (partial rotation).
+
+``stretch`` (factor, original, fast, slow) changes the frequencies for contexts longer than the
+``original`` one: with ``place(turns) = rot_dim * ln(original / (2 pi turns)) / (2 ln theta)``,
+``lo = max(floor(place(fast)), 0)``, ``hi = min(ceil(place(slow)), rot_dim - 1)`` and
+``ramp_j = clamp((j - lo) / max(hi - lo, 0.001), 0, 1)`` pair j turns with
+``f_j / factor * ramp_j + f_j * (1 - ramp_j)``: pairs that turn often within the original context
+keep their frequency, slow ones are slowed by ``factor``, and those between are blended.  Cosine
+and sine are then multiplied by ``0.1 * ln(factor) + 1``.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
 from typing import Optional
+
+import math
 
 import numpy as np
 import torch
@@ -28,7 +38,7 @@ class Rotation:
 
 class RotaryEncoding(PositionEncoding):
     def __init__(self, head_dim: int, theta: float, rot_dim: Optional[int] = None,
-                 pairing: str = "half"):
+                 pairing: str = "half", stretch: Optional[dict] = None):
         if pairing not in ("half", "interleaved"):
             raise ValueError(f"pairing must be 'half' or 'interleaved', got {pairing!r}")
         self.head_dim = head_dim
@@ -37,14 +47,40 @@ class RotaryEncoding(PositionEncoding):
         if self.rot_dim % 2 or not 0 < self.rot_dim <= head_dim:
             raise ValueError(f"rot_dim {self.rot_dim} must be even and at most head_dim {head_dim}")
         self.mode = ops.ROT_HALF if pairing == "half" else ops.ROT_INTERLEAVED
+        self.stretch = None
+        if stretch:
+            self.stretch = {k: float(stretch[k]) for k in ("factor", "original", "fast", "slow")}
+            if (self.stretch["factor"] <= 0.0 or self.stretch["original"] <= 0.0
+                    or self.stretch["fast"] <= 0.0 or self.stretch["slow"] <= 0.0
+                    or self.theta <= 1.0):
+                raise ValueError(f"stretched rotation needs positive numbers and a base above 1, "
+                                 f"got {self.stretch} with base {self.theta}")
         self._rotation: Optional[Rotation] = None
         self._retired = []      # earlier, shorter tables: captured graphs may still read them
 
-    def tables(self, n_positions: int):
+    def frequencies(self):
+        """(float64 frequencies of the pairs, factor on cosine and sine)."""
         half = self.rot_dim // 2
         freq = np.power(self.theta, -2.0 * np.arange(half, dtype=np.float64) / self.rot_dim)
+        st = self.stretch
+        if st is None:
+            return freq, 1.0
+
+        def place(turns: float) -> float:
+            return (self.rot_dim * math.log(st["original"] / (2.0 * math.pi * turns))
+                    / (2.0 * math.log(self.theta)))
+
+        lo = max(math.floor(place(st["fast"])), 0)
+        hi = min(math.ceil(place(st["slow"])), self.rot_dim - 1)
+        ramp = np.clip((np.arange(half, dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return (freq / st["factor"] * ramp + freq * (1.0 - ramp),
+                0.1 * math.log(st["factor"]) + 1.0)
+
+    def tables(self, n_positions: int):
+        freq, factor = self.frequencies()
         ang = np.arange(n_positions, dtype=np.float64)[:, None] * freq[None, :]
-        return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+        return ((np.cos(ang) * factor).astype(np.float32),
+                (np.sin(ang) * factor).astype(np.float32))
 
     def rotation(self, device, max_position: int) -> Rotation:
         """Tables that cover positions 0..max_position; grown in powers of two."""

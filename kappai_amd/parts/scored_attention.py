@@ -6,8 +6,13 @@ multiplied by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at positio
 
     score(i, j) = softcap * tanh(q_i . k_j * scale / softcap) + rel[bucket(i - j), h]
 
-over all ``j <= i`` (or the last ``window``), a softmax whose denominator also holds
-``exp(sink[h])``, the weighted sum of the values, ``W_o``.  ``bucket``: a distance below half the
+over all ``j <= i`` (or the last ``window``; or, with ``chunk``, those ``j <= i`` with
+``floor(j / chunk) = floor(i / chunk)``, chunks counted from position 0 of the sequence), a
+softmax whose denominator also holds ``exp(sink[h])``, the weighted sum of the values, ``W_o``.
+With ``position`` (a rotary encoding) the first places of every q and k head turn by the
+position instead of the norm and the temperature; ``bias``: q, k and v have biases;
+``values_from_keys``: there is no ``W_v``, a kv head's value is its key as projected, before the
+rotation.  ``bucket``: a distance below half the
 table's rows has a row of its own; larger ones share rows on a logarithmic scale that reaches the
 last row at ``bias_max``.  Every piece is optional (``softcap`` 0, no table, no sink, no norm, no
 temperature), so the part also serves designs that use some of them.
@@ -60,7 +65,9 @@ class ScoredAttention(Mixer):
                  whole_qk_norm: bool = False, softcap: float = 0.0,
                  bias_buckets: int = 0, bias_far: float = 0.0, sink: bool = False,
                  temp_coef: float = 0.0, temp_every: int = 1, window: Optional[int] = None,
-                 names=None, weight_suffix: str = ".weight"):
+                 names=None, weight_suffix: str = ".weight", chunk: Optional[int] = None,
+                 position=None, bias: bool = False, bias_suffix: str = ".bias",
+                 values_from_keys: bool = False):
         n = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm",
              "rel": "rel", "sink": "sink"}
         n.update(names or {})
@@ -77,9 +84,24 @@ class ScoredAttention(Mixer):
         self.bias_buckets, self.bias_far, self.has_sink = int(bias_buckets), float(bias_far), sink
         self.temp_coef, self.temp_every = float(temp_coef), int(temp_every)
         self.window = int(window) if window else None
-        self.qkv = Linear([prefix + n["q"], prefix + n["k"], prefix + n["v"]], width,
-                          [num_heads * dim, num_kv_heads * dim, num_kv_heads * vdim],
-                          stage="matmul_qkv", weight_suffix=weight_suffix)
+        self.chunk = int(chunk) if chunk else None
+        if self.window and self.chunk:
+            raise ValueError(f"{prefix}: a sliding window or chunks, not both")
+        self.position, self.values_from_keys = position, bool(values_from_keys)
+        if position is not None and (whole_qk_norm or temp_coef):
+            raise ValueError(f"{prefix}: a rotation goes with neither the whole-projection norm "
+                             "nor the query temperature")
+        if position is not None and position.rot_dim > dim:
+            raise ValueError(f"{prefix}: {position.rot_dim} places turn in heads of {dim}")
+        if self.values_from_keys and vdim != dim:
+            raise ValueError(f"{prefix}: values that are the keys have the keys' size {dim}, "
+                             f"not {vdim}")
+        stacked = ["q", "k"] + ([] if self.values_from_keys else ["v"])
+        sizes = [num_heads * dim, num_kv_heads * dim] + (
+            [] if self.values_from_keys else [num_kv_heads * vdim])
+        self.qkv = Linear([prefix + n[k] for k in stacked], width, sizes, bias=bias,
+                          stage="matmul_qkv", weight_suffix=weight_suffix,
+                          bias_suffix=bias_suffix)
         self._o_name = prefix + n["o"] + weight_suffix
         self.out = Linear([prefix + n["o"]], num_heads * vdim, [width], stage="matmul_attn_out",
                           weight_suffix=weight_suffix)
@@ -94,6 +116,7 @@ class ScoredAttention(Mixer):
                               tuning.LONE_ROWS_FROM if ok and tuning.LONE_ROWS_FROM else None)
 
     def cache_spec(self):
+        # (pages of chunks that lie behind stay with the request: only a window gives them back)
         return PagedKV(self.G, self.head_size, self.window)
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -137,14 +160,23 @@ class ScoredAttention(Mixer):
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")
         with profile.scope("rope_kvput"):
-            q = ops.projection_norm_store(
-                proj, H, G, self.d, self.dv, D, self.q_norm_w, self.k_norm_w, self.norm_eps,
-                self.temp_coef, self.temp_every, k_pool, v_pool, batch.row_pos, batch.row_seg,
-                tables, cache.page_size)
+            if self.position is not None or self.values_from_keys:
+                rot = (self.position.rotation(x.device, batch.max_position)
+                       if self.position is not None else None)
+                q = ops.rotate_widen_store(
+                    proj, H, G, self.d, self.dv, D, rot.cos if rot else None,
+                    rot.sin if rot else None, rot.rot_dim if rot else 0,
+                    rot.mode if rot else ops.ROT_NONE, self.values_from_keys, k_pool, v_pool,
+                    batch.row_pos, batch.row_seg, tables, cache.page_size)
+            else:
+                q = ops.projection_norm_store(
+                    proj, H, G, self.d, self.dv, D, self.q_norm_w, self.k_norm_w, self.norm_eps,
+                    self.temp_coef, self.temp_every, k_pool, v_pool, batch.row_pos,
+                    batch.row_seg, tables, cache.page_size)
         with profile.scope("attn"):
             ctx = ops.paged_attention(q, H, G, D, k_pool, v_pool, batch.row_pos, batch.row_seg,
                                       tables, cache.page_size, self.scale,
-                                      window=self.window or 0,
+                                      window=self.window or 0, chunk=self.chunk or 0,
                                       q_tiles=batch.extra.get("q_tiles"),
                                       single_rows=batch.max_segment_rows == 1,
                                       max_position=batch.max_position,

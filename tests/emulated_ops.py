@@ -156,8 +156,9 @@ def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, e
 
 
 def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, row_seg,
-                    block_tables, page_size, scale, window=0, mods=None, **_unused):
+                    block_tables, page_size, scale, window=0, mods=None, chunk=0, **_unused):
     H, G, d = n_heads, n_kv_heads, head_dim
+    assert not (window and chunk)
     if mods is not None and not mods.active():
         mods = None
     T = q.shape[0]
@@ -165,6 +166,8 @@ def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, r
     for t in range(T):
         p = int(row_pos[t])
         lo = p + 1 - window if window and p + 1 > window else 0
+        if chunk:
+            lo = p - p % chunk
         bt = block_tables[int(row_seg[t])]
         idx = torch.arange(lo, p + 1)
         pages = bt[(idx // page_size).long()].long()
@@ -471,11 +474,11 @@ def latent_store(q, kv, n_heads, dim, rot_dim, rank, head_size, c_norm_w, eps, c
     return out.reshape(T, H * D).to(q.dtype)
 
 
-def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None):
+def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None, out_dtype=None):
     H, n_out, n_in = weight.shape
     T = x.shape[0]
     if out is None:
-        out = torch.empty((T, H * n_out), dtype=x.dtype)
+        out = torch.empty((T, H * n_out), dtype=out_dtype or x.dtype)
         out_head_stride = n_out
     for h in range(H):
         xi = x[:, h * x_head_stride:h * x_head_stride + n_in].to(F32)
@@ -488,7 +491,8 @@ CONV_SILU_MAX_TAPS = 17
 GATE_SILU, GATE_SIGMOID = 0, 1
 
 
-def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot):
+def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot, bias=None,
+              activation=True):
     C, n = taps.shape
     xf = x[:, :C].to(F32)
     out = torch.empty((x.shape[0], C), dtype=F32)
@@ -500,7 +504,9 @@ def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot):
             acc = torch.zeros(C)
             for j in range(n):
                 acc = acc + taps[:, j] * seq[i + j]
-            out[t0 + i] = acc * torch.sigmoid(acc)
+            if bias is not None:
+                acc = acc + bias
+            out[t0 + i] = acc * torch.sigmoid(acc) if activation else acc
         if n > 1:
             state[slot] = seq[-(n - 1):]
     return out.to(x.dtype)
@@ -508,21 +514,34 @@ def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot):
 
 def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_bias, z_sign,
                             q_scale, state, seg_start, seg_pos0, seg_slot, beta=None,
-                            unit_qk=False, unit_eps=1e-6, form="auto"):
+                            unit_qk=False, unit_eps=1e-6, form="auto", decay="softplus",
+                            bonus=None, silu_inputs=False):
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     T = q.shape[0]
-    qf = q[:, :Hk * d].to(F32).reshape(T, Hk, d)
-    kf = k[:, :Hk * d].to(F32).reshape(T, Hk, d)
+
+    def taken(x):
+        if not silu_inputs:
+            return x.to(F32)
+        x = x.to(F32)
+        return (x * torch.sigmoid(x)).to(q.dtype).to(F32)       # rounded as it is stored
+
+    qf = taken(q[:, :Hk * d]).reshape(T, Hk, d)
+    kf = taken(k[:, :Hk * d]).reshape(T, Hk, d)
     if unit_qk:
         qf = qf / torch.sqrt((qf * qf).sum(-1, keepdim=True) + unit_eps)
         kf = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + unit_eps)
     qf = (qf * q_scale).repeat_interleave(H // Hk, dim=1)
     kf = kf.repeat_interleave(H // Hk, dim=1)
-    vf = v[:, :H * dv].to(F32).reshape(T, H, dv)
-    zz = z[:, :H * d].to(F32)
-    if z_bias is not None:
-        zz = zz + z_bias
-    a = torch.exp(-rate[:, None] * torch.nn.functional.softplus(z_sign * zz.reshape(T, H, d)))
+    vf = taken(v[:, :H * dv]).reshape(T, H, dv)
+    if decay == "fixed":
+        a = rate[None, :, None].expand(T, H, d)
+    else:
+        zz = z[:, :H * d].to(F32)
+        if z_bias is not None:
+            zz = zz + z_bias
+        zz = zz.reshape(T, H, d)
+        a = (torch.exp(-torch.exp(zz)) if decay == "double_exp" else
+             torch.exp(-rate[:, None] * torch.nn.functional.softplus(z_sign * zz)))
     b = torch.sigmoid(beta[:, :H].to(F32)) if beta is not None else None
     out = torch.empty((T, H, dv), dtype=F32)
     for s in range(seg_slot.shape[0]):
@@ -530,6 +549,11 @@ def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_
         S = (torch.zeros((H, d, dv)) if int(seg_pos0[s]) == 0
              else state[slot].transpose(1, 2).clone())
         for t in range(t0, t1):
+            if bonus is not None:
+                kv = kf[t][:, :, None] * vf[t][:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", S + bonus[:, :, None] * kv, qf[t])
+                S = a[t][:, :, None] * S + kv
+                continue
             S = a[t][:, :, None] * S
             if b is not None:
                 u = b[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
@@ -545,11 +569,86 @@ def head_norm_gate(o, weight, eps, gate, gate_kind, n_heads, vdim, out_dtype):
     H, dv = n_heads, vdim
     T = o.shape[0]
     x = o.reshape(T, H, dv)
-    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight        # [dv] or [H, dv]
     g = gate[:, :H * dv].to(F32).reshape(T, H, dv)
     g = g * torch.sigmoid(g) if gate_kind == GATE_SILU else torch.sigmoid(g)
     return (x * g).reshape(T, H * dv).to(out_dtype)
 
+
+
+def rotate_widen_store(proj, n_heads, n_kv_heads, dim, vdim, head_size, cos, sin, rot_dims,
+                       rot_mode, values_are_keys, k_pool, v_pool, row_pos, row_seg, block_tables,
+                       page_size):
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    T = proj.shape[0]
+    p = proj.to(F32)
+    pos = row_pos.long()
+    q = p[:, :H * d].reshape(T, H, d)
+    k = p[:, H * d:(H + G) * d].reshape(T, G, d)
+    v = k if values_are_keys else p[:, (H + G) * d:(H + G) * d + G * dv].reshape(T, G, dv)
+    qo, ko, vo = (torch.zeros((T, n, D), dtype=F32) for n in (H, G, G))
+    qo[:, :, :d] = _rotate(q, pos, cos, sin, rot_dims, rot_mode)
+    ko[:, :, :d] = _rotate(k, pos, cos, sin, rot_dims, rot_mode)
+    vo[:, :, :dv] = v
+    _store(k_pool, v_pool, ko, vo, row_pos, row_seg, block_tables, page_size)
+    return qo.reshape(T, H * D).to(proj.dtype)
+
+
+def token_shift_mix(h, mu, state, row_pos, row_seg, seg_start, seg_slot):
+    T, W = h.shape
+    hf = h.to(F32)
+    before = torch.zeros((T, W), dtype=F32)
+    for s in range(seg_slot.shape[0]):
+        t0, t1, slot = int(seg_start[s]), int(seg_start[s + 1]), int(seg_slot[s])
+        if t1 <= t0:
+            continue
+        if int(row_pos[t0]) > 0:
+            before[t0] = state[slot]
+        before[t0 + 1:t1] = hf[t0:t1 - 1]
+        state[slot] = hf[t1 - 1]
+    return (hf[None] + (before - hf)[None] * mu[:, None, :]).to(h.dtype)
+
+
+def tanh(x):
+    return torch.tanh(x.to(F32)).to(x.dtype)
+
+
+def gated_unit_scan(gates, gate_bias, u, y, softplus_lam, rate, state, seg_start, seg_pos0,
+                    seg_slot, chunks=None, seg_chunk0=None):
+    T, W = u.shape
+    g = gates + gate_bias
+    a = torch.exp(-rate * torch.sigmoid(g[:, :W]) * softplus_lam)
+    b = torch.sqrt(torch.clamp(1.0 - a * a, min=0.0)) * torch.sigmoid(g[:, W:]) * u.to(F32)
+    z = y[:, :W].to(F32)
+    gate = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+    out = torch.empty((T, W), dtype=F32)
+    for s in range(seg_slot.shape[0]):
+        t0, t1, slot = int(seg_start[s]), int(seg_start[s + 1]), int(seg_slot[s])
+        S = torch.zeros(W) if int(seg_pos0[s]) == 0 else state[slot].clone()
+        for t in range(t0, t1):
+            S = a[t] * S + b[t]
+            out[t] = S * gate[t]
+        state[slot] = S
+    return out.to(u.dtype)
+
+
+def pair_norm_sum(a, b, scale_a=1.0, scale_b=1.0, weight_a=None, weight_b=None, eps=0.0):
+    def side(x, w):
+        x = x.to(F32)
+        if w is None:
+            return x
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w
+
+    return scale_a * side(a, weight_a) + scale_b * side(b, weight_b)
+
+
+def stream_enter(resid, delta, again, row):
+    if delta is not None:
+        resid.add_(delta.to(F32))
+    if again is not None:
+        resid.add_(again)
+    if row is not None:
+        resid.add_(row)
 
 
 class _Plan:
@@ -595,7 +694,8 @@ def moe_combine(y, weights, plan):
 ALL = ["add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
        "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
        "output_norm_add", "projection_norm_store", "latent_store", "headwise_linear", "conv_silu",
-       "matrix_state_recurrence", "head_norm_gate",
+       "matrix_state_recurrence", "head_norm_gate", "rotate_widen_store", "token_shift_mix", "tanh",
+       "gated_unit_scan", "pair_norm_sum", "stream_enter",
        "embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
