@@ -62,15 +62,13 @@ def _chunked_attention(left: KeyReader, where: str, values_are_keys: bool) -> Di
     out = {"heads": left.int("heads"), "kv_heads": left.int("kv_heads"), "dim": left.int("dim"),
            "scale": left.float("scale"), "rot_base": rot.float("base"),
            "rot_dims": rot.int("dims"), "stretch": None, "chunk": mask.int("size")}
-    out["vdim"] = left.int("vdim", out["dim"]) if values_are_keys else left.int("vdim")
+    # (values that are the keys have the keys' size, whatever the file says of them)
+    out["vdim"] = out["dim"] if values_are_keys else left.int("vdim")
     _positive(where + " left", heads=out["heads"], kv_heads=out["kv_heads"], dim=out["dim"],
               vdim=out["vdim"])
     if out["heads"] % out["kv_heads"]:
         raise ConfigError(f"{where}: {out['heads']} heads cannot be shared out over "
                           f"{out['kv_heads']} kv heads")
-    if values_are_keys and out["vdim"] != out["dim"]:
-        raise ConfigError(f"{where}: mixer.left.vdim ({out['vdim']}) must equal mixer.left.dim "
-                          f"({out['dim']}): the values are the keys")
     if out["rot_dims"] < 0 or out["rot_dims"] % 2 or out["rot_dims"] > out["dim"]:
         raise ConfigError(f"{where}: mixer.left.rot.dims ({out['rot_dims']}) must be even and at "
                           f"most mixer.left.dim ({out['dim']})")
