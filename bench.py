@@ -108,7 +108,11 @@ COMPARISONS = {"w1024": ("dapipel-w1024", "lfm2-like-w1024"),
                # the Dukolorn decoder beside the same LFM2 shapes (its closest relative: a hybrid
                # of recurrent and attention layers with SiLU-gated dense feed-forwards)
                "dukolorn-w1024": ("dukolorn-w1024", "lfm2-like-w1024"),
-               "dukolorn-w2048": ("dukolorn-w2048", "lfm2-like-w2048")}
+               "dukolorn-w2048": ("dukolorn-w2048", "lfm2-like-w2048"),
+               # the Zumuzen decoder beside them as well (pairs of mixers where the LFM2 shapes
+               # have attention, a gated recurrence per channel where they have convolutions)
+               "zumuzen-w1024": ("zumuzen-w1024", "lfm2-like-w1024"),
+               "zumuzen-w2048": ("zumuzen-w2048", "lfm2-like-w2048")}
 
 
 def stage_table(runner, entries_of, reps):
@@ -567,14 +571,14 @@ def main() -> int:
                     help="serving workloads: a repeat penalty over the last 64 tokens before "
                          "the greedy choice (1: none)")
     ap.add_argument("--compare", default="", metavar="SIZES",
-                    help="instead of the headline run: prompt and decode steps of the Dapipel or "
-                         "Dukolorn decoder beside the LFM2 shape of equal size, at these sizes (comma "
+                    help="instead of the headline run: prompt and decode steps of the Dapipel, "
+                         "Dukolorn or Zumuzen decoder beside the LFM2 shape of equal size, at these sizes (comma "
                          "separated: " + ", ".join(sorted(COMPARISONS)) + "; 'all')")
     args = ap.parse_args()
     if args.compare:
         keys = (sorted(k for k in COMPARISONS if k.startswith("w")) if args.compare == "all"
-                else sorted(k for k in COMPARISONS if k.startswith("dukolorn"))
-                if args.compare == "dukolorn" else args.compare.split(","))
+                else sorted(k for k in COMPARISONS if k.startswith(args.compare + "-"))
+                if args.compare in ("dukolorn", "zumuzen") else args.compare.split(","))
         for k in keys:
             if k not in COMPARISONS:
                 print(f"bench.py: no comparison {k!r}; known: {', '.join(sorted(COMPARISONS))}")

@@ -151,6 +151,54 @@ SHAPES.update({
 })
 
 
+def _zumuzen(width, mixers, heads, kv_heads, dim, chunk, l_heads, l_dim, l_vdim, t_heads, t_dim,
+             inner, blocks, ff, vocab=65536, rank=64, taps=4, loop=None) -> dict:
+    """Layers by letter: "p" a softmax attention over chunks beside a linear attention with a
+    fixed decay a head, "t" a softmax attention over chunks whose values are its keys (stretched
+    frequencies, a sink) beside a time mixing with a bonus, "r" a real-gated unit; dense
+    feed-forwards of ``ff`` everywhere."""
+    layers = []
+    for kind in mixers:
+        left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                "scale": dim ** -0.5, "rot": {"base": 10000.0, "dims": dim},
+                "mask": {"size": chunk}}
+        if kind == "p":
+            decay = [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, l_heads - 1)) for h in range(l_heads)]
+            mixer = {"left": left, "right": {"heads": l_heads, "dim": l_dim, "vdim": l_vdim,
+                                             "decay": decay}}
+            layers.append({"type": "parallel", "mixer": mixer})
+        elif kind == "t":
+            left["rot"]["scaling"] = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+            mixer = {"left": left, "right": {"heads": t_heads, "dim": t_dim, "decay_rank": rank},
+                     "left_scale": 1.0, "right_scale": 1.0}
+            layers.append({"type": "parallel_2", "mixer": mixer})
+        else:
+            layers.append({"type": "rglru", "mixer": {"width": inner, "blocks": blocks,
+                                                      "conv": taps}})
+        layers[-1]["mlp"] = {"kind": "dense", "ff": ff}
+    out = {"architecture": "Zumuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+           "layers": layers}
+    if loop is not None:
+        out["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return out
+
+
+SHAPES.update({
+    # eight layers at a width of 1024: a pair of mixers where the LFM2 pattern has attention (2,
+    # 5, 7; 16 heads of 64 on 4 kv heads in chunks of 1024), a real-gated unit of 1024 channels
+    # in 8 blocks elsewhere; 8 linear-attention heads of 64 x 64, 16 time-mixing heads of 64
+    "zumuzen-w1024": _zumuzen(1024, "rrprrtrp", 16, 4, 64, 1024, 8, 64, 64, 16, 64, 1024, 8,
+                              4608),
+    # the same at a width of 2048: 32 heads on 8 kv heads in chunks of 2048, linear-attention
+    # heads of 64 x 128, 32 time-mixing heads of 64, 2048 channels in 16 blocks
+    "zumuzen-w2048": _zumuzen(2048, "rrprrtrp", 32, 8, 64, 2048, 16, 64, 128, 32, 64, 2048, 16,
+                              8192),
+    # a tiny one for smoke runs: the last two layers are passed twice
+    "zumuzen-tiny": _zumuzen(64, "prt", 4, 2, 8, 24, 2, 8, 16, 2, 16, 48, 3, 96, vocab=256,
+                             rank=4, taps=3, loop=(1, 3, 2)),
+})
+
+
 def named_shape(name: str) -> dict:
     """A copy of the configuration called ``name`` (any case), or a ``KeyError`` naming them all."""
     key = name.strip().lower()

@@ -671,6 +671,215 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
 }
 
 // ---------------------------------------------------------------------------------------
+// One fixed decay a head, S <- lam S + k v^T, o = S^T q, over long portions in chunks of rows.
+// A constant decay has a form without a chain along the tokens and without a division: inside
+// a chunk of n rows  o_i = sum_(j <= i) lam^(i - j) (q_i . k_j) v_j + lam^(i + 1) S0^T q_i  with
+// S0 the state the chunk starts from, and behind it  S = lam^n S0 + sum_j lam^(n - 1 - j) k_j
+// v_j^T.  Every power is of a number in [0, 1] with an exponent >= 0.  Three passes, as the scans
+// per channel take them: the chunks' own sums side by side; a thread an element of the state
+// carries it over a segment's chunks in order, leaving in `carry` the state every chunk starts
+// from; the chunks' outputs side by side.  Everything is float32 on the vector units (scores,
+// their weights and the state are asked for in 32 bits): products of tiles staged in LDS so that
+// the summed index is the row of both operands, a thread keeping 4 x 4 results.
+// `carry` [n_chunks, H, dv, d] (a head's matrix column by column, as the state).
+// ---------------------------------------------------------------------------------------
+#define FD_C 32         // most rows of a chunk
+#define FD_T 64         // key channels / value channels a tile
+#define FD_THREADS 128
+#define FD_CS (FD_C + 4)   // row strides in LDS: multiples of four floats, off the powers of two
+#define FD_TS (FD_T + 4)
+
+// acc[a][b] += sum_(k < kn) X[k][a0 + a] * Y[k][b0 + b]
+__device__ __forceinline__ void fd_outer(float (&acc)[4][4], const float* X, int xs, const float* Y,
+                                         int ys, int a0, int b0, int kn) {
+  for (int k = 0; k < kn; ++k) {
+    const float4 x4 = *reinterpret_cast<const float4*>(X + k * xs + a0);
+    const float4 y4 = *reinterpret_cast<const float4*>(Y + k * ys + b0);
+    const float x[4] = {x4.x, x4.y, x4.z, x4.w}, y[4] = {y4.x, y4.y, y4.z, y4.w};
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(x[a], y[b], acc[a][b]);
+  }
+}
+
+template <typename TV>
+__global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_sums_kernel(
+    const float* __restrict__ kf, const TV* __restrict__ v, int v_stride,
+    const float* __restrict__ rate, const int* __restrict__ chunks, int H, int d, int dv,
+    int n_ct, float* __restrict__ carry) {
+  __shared__ __attribute__((aligned(16))) float Ks[FD_C][FD_T];
+  __shared__ __attribute__((aligned(16))) float Vs[FD_C][FD_T];
+  __shared__ float pw[FD_C + 1];
+  const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int c0 = (blockIdx.z % n_ct) * FD_T, r0 = (blockIdx.z / n_ct) * FD_T;
+  const int row0 = chunks[3 * ch + 1], n = min(chunks[3 * ch + 2], FD_C);
+  if (tid <= FD_C) pw[tid] = powf(rate[h], (float)tid);
+  __syncthreads();
+  for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+    const int j = i / FD_T, e = i % FD_T;
+    const size_t row = (size_t)(row0 + j);
+    Ks[j][e] = (j < n && r0 + e < d) ? kf[(row * H + h) * d + r0 + e] * pw[n - 1 - j] : 0.f;
+    Vs[j][e] = (j < n && c0 + e < dv) ? to_f32(v[row * v_stride + (size_t)h * dv + c0 + e]) : 0.f;
+  }
+  __syncthreads();
+  for (int tile = tid; tile < (FD_T / 4) * (FD_T / 4); tile += FD_THREADS) {
+    const int a0 = (tile / (FD_T / 4)) * 4, b0 = (tile % (FD_T / 4)) * 4;
+    float acc[4][4] = {};
+    fd_outer(acc, &Vs[0][0], FD_T, &Ks[0][0], FD_T, a0, b0, n);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int c = c0 + a0 + a, r = r0 + b0 + b;
+        if (c < dv && r < d) carry[(((size_t)ch * H + h) * dv + c) * d + r] = acc[a][b];
+      }
+  }
+}
+
+__global__ __launch_bounds__(256) void fixed_decay_chunk_carry_kernel(
+    const float* __restrict__ rate, const int* __restrict__ chunks,
+    const int* __restrict__ seg_chunk0, const int* __restrict__ seg_pos0,
+    const int* __restrict__ seg_slot, int H, int d, int dv, float* __restrict__ carry,
+    float* __restrict__ state) {
+  const int seg = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x, n_el = dv * d;
+  if (e >= n_el) return;
+  const int ch0 = seg_chunk0[seg], ch1 = seg_chunk0[seg + 1];
+  if (ch0 >= ch1) return;
+  const float lam = rate[h], lam_full = powf(lam, (float)FD_C);
+  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + e;
+  float S = seg_pos0[seg] > 0 ? *st : 0.f;
+  for (int c = ch0; c < ch1; c += 4) {
+    float own[4];
+    int rows[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int cc = min(c + i, ch1 - 1);
+      own[i] = carry[((size_t)cc * H + h) * n_el + e];
+      rows[i] = chunks[3 * cc + 2];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (c + i >= ch1) break;
+      carry[((size_t)(c + i) * H + h) * n_el + e] = S;      // the state the chunk starts from
+      S = fmaf(rows[i] == FD_C ? lam_full : powf(lam, (float)rows[i]), S, own[i]);
+    }
+  }
+  *st = S;
+}
+
+template <typename TV>
+__global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_out_kernel(
+    const float* __restrict__ qf, const float* __restrict__ kf, const TV* __restrict__ v,
+    int v_stride, const float* __restrict__ rate, const int* __restrict__ chunks, int H, int d,
+    int dv, const float* __restrict__ carry, float* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) float Qt[FD_T][FD_CS];     // [key channel][row]
+  __shared__ __attribute__((aligned(16))) float Kt[FD_T][FD_CS];
+  __shared__ __attribute__((aligned(16))) float Pt[FD_C][FD_CS];     // [key row j][query row i]
+  __shared__ __attribute__((aligned(16))) float Vs[FD_C][FD_T];      // [row][value channel]
+  __shared__ __attribute__((aligned(16))) float St[FD_T][FD_TS];     // [key channel][value channel]
+  __shared__ float pw[FD_C + 1];
+  const int ch = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * FD_T, tid = threadIdx.x;
+  const int row0 = chunks[3 * ch + 1], n = min(chunks[3 * ch + 2], FD_C);
+  if (tid <= FD_C) pw[tid] = powf(rate[h], (float)tid);
+  // the scores of the chunk, P[i][j] = q_i . k_j: 64 tiles of 4 x 4, one wave
+  const int pi0 = (tid / (FD_C / 4)) * 4, pj0 = (tid % (FD_C / 4)) * 4;
+  float accP[4][4] = {};
+  for (int r0 = 0; r0 < d; r0 += FD_T) {
+    __syncthreads();
+    for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+      const int j = i / FD_T, e = i % FD_T;
+      const bool ok = j < n && r0 + e < d;
+      const size_t at = ((size_t)(row0 + j) * H + h) * d + r0 + e;
+      Qt[e][j] = ok ? qf[at] : 0.f;
+      Kt[e][j] = ok ? kf[at] : 0.f;
+    }
+    __syncthreads();
+    if (tid < (FD_C / 4) * (FD_C / 4))
+      fd_outer(accP, &Qt[0][0], FD_CS, &Kt[0][0], FD_CS, pi0, pj0, min(FD_T, d - r0));
+  }
+  if (tid < (FD_C / 4) * (FD_C / 4)) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int i = pi0 + a, j = pj0 + b;
+        Pt[j][i] = (j <= i && i < n) ? accP[a][b] * pw[i - j] : 0.f;
+      }
+  }
+  for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+    const int j = i / FD_T, e = i % FD_T;
+    Vs[j][e] = (j < n && c0 + e < dv)
+                   ? to_f32(v[(size_t)(row0 + j) * v_stride + (size_t)h * dv + c0 + e]) : 0.f;
+  }
+  __syncthreads();
+  // the outputs, 32 rows x 64 value channels: 128 tiles of 4 x 4
+  const int oi0 = (tid / (FD_T / 4)) * 4, oc0 = (tid % (FD_T / 4)) * 4;
+  float accO[4][4] = {}, accS[4][4] = {};
+  fd_outer(accO, &Pt[0][0], FD_CS, &Vs[0][0], FD_T, oi0, oc0, n);
+  const float* S0 = carry + ((size_t)ch * H + h) * dv * d;
+  for (int r0 = 0; r0 < d; r0 += FD_T) {
+    __syncthreads();
+    for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+      const int j = i / FD_T, e = i % FD_T;
+      Qt[e][j] = (j < n && r0 + e < d) ? qf[((size_t)(row0 + j) * H + h) * d + r0 + e] : 0.f;
+    }
+    for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
+      const int c = i / FD_T, e = i % FD_T;
+      St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(c0 + c) * d + r0 + e] : 0.f;
+    }
+    __syncthreads();
+    fd_outer(accS, &Qt[0][0], FD_CS, &St[0][0], FD_TS, oi0, oc0, min(FD_T, d - r0));
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int i = oi0 + a;
+    if (i >= n) continue;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int c = c0 + oc0 + b;
+      if (c < dv)
+        out[((size_t)(row0 + i) * H + h) * dv + c] = fmaf(pw[i + 1], accS[a][b], accO[a][b]);
+    }
+  }
+}
+
+// qf, kf [T, H, d] float32 as recurrence_prep leaves them, v [T, >= H dv] with a row stride,
+// rate [H] the decays, chunks [n_chunks, 3] = (segment, first row, rows <= 32), seg_chunk0
+// [S + 1], carry [n_chunks, H, dv, d] floats of scratch, state [slots, H, dv, d], out [T, H dv].
+extern "C" int kappai_fixed_decay_chunks(const float* qf, const float* kf, const void* v,
+                                         int v_stride, int v_is_bf16, const float* rate,
+                                         float* state, const int* seg_pos0, const int* seg_slot,
+                                         const int* chunks, const int* seg_chunk0, int n_chunks,
+                                         int chunk_rows, int T, int S, int H, int d, int dv,
+                                         float* carry, float* out, hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (H < 1 || H > 65535 || d < 1 || dv < 1 || n_chunks < 1 ||
+      chunk_rows < 1 || chunk_rows > FD_C || !chunks || !seg_chunk0 || !carry || !rate)
+    return (int)hipErrorInvalidValue;
+  const int n_ct = (dv + FD_T - 1) / FD_T, n_rt = (d + FD_T - 1) / FD_T;
+  const int el_blocks = (dv * d + 255) / 256;
+  if (n_ct * n_rt > 65535 || el_blocks > 65535) return (int)hipErrorInvalidValue;
+  const dim3 sums(n_chunks, H, n_ct * n_rt), outs(n_chunks, H, n_ct);
+  if (v_is_bf16)
+    hipLaunchKernelGGL(fixed_decay_chunk_sums_kernel<bf16_t>, sums, dim3(FD_THREADS), 0, stream,
+                       kf, (const bf16_t*)v, v_stride, rate, chunks, H, d, dv, n_ct, carry);
+  else
+    hipLaunchKernelGGL(fixed_decay_chunk_sums_kernel<float>, sums, dim3(FD_THREADS), 0, stream,
+                       kf, (const float*)v, v_stride, rate, chunks, H, d, dv, n_ct, carry);
+  hipLaunchKernelGGL(fixed_decay_chunk_carry_kernel, dim3(S, H, el_blocks), dim3(256), 0, stream,
+                     rate, chunks, seg_chunk0, seg_pos0, seg_slot, H, d, dv, carry, state);
+  if (v_is_bf16)
+    hipLaunchKernelGGL(fixed_decay_chunk_out_kernel<bf16_t>, outs, dim3(FD_THREADS), 0, stream,
+                       qf, kf, (const bf16_t*)v, v_stride, rate, chunks, H, d, dv, carry, out);
+  else
+    hipLaunchKernelGGL(fixed_decay_chunk_out_kernel<float>, outs, dim3(FD_THREADS), 0, stream,
+                       qf, kf, (const float*)v, v_stride, rate, chunks, H, d, dv, carry, out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // Per head: o / sqrt(mean(o^2) + eps) * weight[dv] * gate, gate = silu(g) (kind 0) or sigmoid(g)
 // (kind 1) of the projection g [T, >= H dv] with a row stride.  A wave a (row, head).
 // weight_stride: 0 when the heads share one weight [dv], dv when each has its own [H, dv].

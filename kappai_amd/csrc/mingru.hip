@@ -50,8 +50,10 @@ __device__ __forceinline__ void scan_terms(const scan_in<TP>& in, int W, int t, 
   } else {
     const float* gp = in.gates + (size_t)t * 2 * W + c;
     const float uu = to_f32(in.u[(size_t)t * W + c]);
-    a = expf(-in.rate * sigmoid_f(gp[0] + in.gate_bias[c]) * in.sp[c]);
-    b = sqrtf(fmaxf(1.0f - a * a, 0.f)) * sigmoid_f(gp[W] + in.gate_bias[W + c]) * uu;
+    // (1 - a^2 from the logarithm: a decay close to one loses nothing to cancellation)
+    const float la = -in.rate * sigmoid_f(gp[0] + in.gate_bias[c]) * in.sp[c];
+    a = expf(la);
+    b = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f)) * sigmoid_f(gp[W] + in.gate_bias[W + c]) * uu;
     if (OUT) {
       const float z = to_f32(in.proj[(size_t)t * in.y_stride + c]);
       g = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));

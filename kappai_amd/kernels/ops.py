@@ -1997,6 +1997,7 @@ SCAN_FORMS = {"auto": 0, "wave": 1, "block": 2}
 
 
 DECAY_KINDS = {"softplus": 0, "double_exp": 1, "fixed": 2}
+FIXED_DECAY_CHUNK_ROWS = 32     # the most rows of a chunk the chunked form of a fixed decay takes
 
 
 def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
@@ -2009,7 +2010,9 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                             beta: Optional[torch.Tensor] = None, unit_qk: bool = False,
                             unit_eps: float = 1e-6, form: str = "auto",
                             decay: str = "softplus", bonus: Optional[torch.Tensor] = None,
-                            silu_inputs: bool = False) -> torch.Tensor:
+                            silu_inputs: bool = False, chunks: Optional[torch.Tensor] = None,
+                            seg_chunk0: Optional[torch.Tensor] = None,
+                            chunk_rows: int = 0) -> torch.Tensor:
     """A state ``S`` [dim, vdim] per head, float32, kept column by column in ``state``
     [slots, H, vdim, dim] (a segment that starts at position 0 starts from zero).  Per token, with the decay per key channel
     ``a = exp(-rate[h] * softplus(z_sign * (z + z_bias)))``:
@@ -2028,7 +2031,11 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     projections and the result is float32.  Returns ``o`` [T, H vdim] float32.
 
     ``form`` = "wave" | "block" forces one of the two kernels (for tests): a wave that reads each
-    token from global memory, or a block of waves that takes the tokens in chunks through LDS."""
+    token from global memory, or a block of waves that takes the tokens in chunks through LDS.
+
+    ``chunks`` [n, 3] = (segment, first row, rows <= ``chunk_rows`` <= 32) with ``seg_chunk0``
+    [S + 1], as for ``mingru_scan``: a fixed decay (no ``beta``, no ``bonus``, H == Hk) is then
+    worked chunk by chunk in three passes, with no chain along the tokens of a chunk."""
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     _need(form in SCAN_FORMS, lambda: f"matrix_state_recurrence: form {form!r}")
     _need(decay in DECAY_KINDS and (z is None) == (decay == "fixed")
@@ -2084,6 +2091,22 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     out = torch.empty((T, H * dv), dtype=F32, device=dev)
     values = vf if silu_inputs else v
     mode = 1 if beta is not None else 2 if bonus is not None else 0
+    if chunks is not None and decay == "fixed" and mode == 0 and H == Hk:
+        _gpu("chunks", chunks, I32)
+        _gpu("seg_chunk0", seg_chunk0, I32)
+        _need(chunks.dim() == 2 and chunks.shape[1] == 3 and seg_chunk0.shape[0] == S + 1
+              and 1 <= chunk_rows <= FIXED_DECAY_CHUNK_ROWS,
+              lambda: f"matrix_state_recurrence: chunk tables {tuple(chunks.shape)} of "
+                      f"{chunk_rows} rows do not fit")
+        n_chunks = chunks.shape[0]
+        carry = torch.empty((n_chunks, H, dv, d), dtype=F32, device=dev)
+        check(lib.kappai_fixed_decay_chunks(
+            _ptr(qf), _ptr(kf), _ptr(values), _c_int(values.stride(0)),
+            _c_int(_is_bf16(values.dtype)), _ptr(rate), _ptr(state), _ptr(seg_pos0),
+            _ptr(seg_slot), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks), _c_int(chunk_rows),
+            _c_int(T), _c_int(S), _c_int(H), _c_int(d), _c_int(dv), _ptr(carry), _ptr(out),
+            _stream()), "fixed_decay_chunks")
+        return out
     check(lib.kappai_matrix_state_scan(
         _ptr(qf), _ptr(kf), _ptr(af), _ptr(bonus if bonus is not None else bf), _ptr(values),
         _c_int(values.stride(0)),

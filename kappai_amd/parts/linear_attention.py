@@ -37,10 +37,11 @@ from typing import Dict, List
 import torch
 
 from ..cache.specs import CacheBundle, FixedState
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, INIT_SMALL, VECTOR, TensorSpec
 from .base import Mixer, register_part
 from .linear import Linear
+from .mingru import ScanChunks
 
 
 def _columns(proj: torch.Tensor, start: int, n: int) -> torch.Tensor:
@@ -135,6 +136,10 @@ class FixedDecayAttention(Mixer):
         self._norm = prefix + n["norm"]
         self.norm_w = self.rate = None
 
+    @property
+    def step_tables(self) -> ScanChunks:
+        return ScanChunks(min(tuning.SCAN_CHUNK_ROWS, ops.FIXED_DECAY_CHUNK_ROWS))
+
     def cache_spec(self):
         return FixedState((self.H, self.dv, self.d), "float32")
 
@@ -155,11 +160,16 @@ class FixedDecayAttention(Mixer):
         H, d, dv = self.H, self.d, self.dv
         proj = self.inputs.forward(x)
         o_k, o_v, o_g = H * d, 2 * H * d, 2 * H * d + H * dv
+        # long portions: the decay is a constant, so a chunk of rows needs no chain along them
+        chunked = batch.max_segment_rows > tuning.SCAN_CHUNKS_FROM_ROWS
         with profile.scope("scan"):
             o = ops.matrix_state_recurrence(
                 proj, proj[:, o_k:], proj[:, o_v:], None, H, H, d, dv, self.rate, None, 1.0, 1.0,
                 cache.state, batch.seg_start, batch.seg_pos0, batch.seg_slot, decay="fixed",
-                silu_inputs=True)
+                silu_inputs=True,
+                chunks=batch.extra.get("scan_chunks") if chunked else None,
+                seg_chunk0=batch.extra.get("scan_seg_chunk0") if chunked else None,
+                chunk_rows=min(tuning.SCAN_CHUNK_ROWS, ops.FIXED_DECAY_CHUNK_ROWS))
             # (all heads are normed together: one "head" of H * dv for the kernel)
             y = ops.head_norm_gate(o, self.norm_w, self.norm_eps, proj[:, o_g:],
                                    ops.GATE_SIGMOID, 1, H * dv, self.dtype)

@@ -515,7 +515,8 @@ def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot, b
 def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_bias, z_sign,
                             q_scale, state, seg_start, seg_pos0, seg_slot, beta=None,
                             unit_qk=False, unit_eps=1e-6, form="auto", decay="softplus",
-                            bonus=None, silu_inputs=False):
+                            bonus=None, silu_inputs=False, chunks=None, seg_chunk0=None,
+                            chunk_rows=0):
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     T = q.shape[0]
 

@@ -153,7 +153,7 @@ def test_the_order_of_the_calls_and_what_they_ask_of_the_cache_manager():
 
 @pytest.mark.parametrize("base,dims,stretch", [
     (3000.0, 16, (4.0, 64, 8.0, 1.0)), (5000.0, 40, (8.0, 32, 1000.0, 0.001)),
-    (250000.0, 32, (2.0, 512, 32.0, 1.0)), (10000.0, 64, (1.0, 4096, 32.0, 1.0)),
+    (300000.0, 24, (3.0, 256, 16.0, 2.0)), (10000.0, 64, (1.0, 4096, 32.0, 1.0)),
     (100.0, 8, (16.0, 16, 2.0, 2.0)), (9000.0, 8, None)])
 def test_stretched_frequencies(base, dims, stretch):
     """The encoding's tables against the plain statement: unstretched pairs, slowed pairs and

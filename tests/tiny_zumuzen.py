@@ -149,9 +149,11 @@ FP32_TOL = 3e-5
 def assert_matches_plain(got, model_dir, requests, dtype, what=""):
     """float32: every row within FP32_TOL.  bfloat16: against what rounding the same values to
     bfloat16 costs the plain implementation itself.  Its root mean square row error is the yard:
-    no row over six yards and at most one row in fifty over three, but for rows where the plain
-    implementation's own rounding error is that large too (there a row may err by half as much
-    again as the plain one)."""
+    no row over six yards and at most one row in fifty over three.  Rows that rounding alone
+    moves by more than two yards in the plain implementation are badly conditioned (a head's
+    read-out that nearly cancels before it is divided by its root mean square, say): the error
+    there is a draw from a wide spread, so such a row may err by eight times the plain one's own
+    error."""
     ref = plain_logits(model_dir, requests)
     errs = row_errors(got, ref)
     worst = max(errs, key=errs.get)
@@ -161,7 +163,12 @@ def assert_matches_plain(got, model_dir, requests, dtype, what=""):
     own = row_errors({k: plain_logits(model_dir, requests, torch.bfloat16)[k[0]][k[1]]
                       for k in got}, ref)
     yard = float(np.sqrt(np.mean(np.square(list(own.values())))))
-    bad = [k for k, e in errs.items() if e > max(6 * yard, 1.5 * own[k])]
-    over = [k for k, e in errs.items() if e > max(3 * yard, 1.5 * own[k])]
+    touchy = {k for k in errs if own[k] > 2 * yard}
+
+    def bound(k, yards):
+        return max(yards * yard, 8.0 * own[k] if k in touchy else 1.5 * own[k])
+
+    bad = [k for k, e in errs.items() if e > bound(k, 6)]
+    over = [k for k, e in errs.items() if e > bound(k, 3)]
     assert not bad, (what, bad[:5], [errs[k] for k in bad[:5]], yard)
     assert len(over) <= max(1, len(errs) // 50), (what, len(over), len(errs), yard, over[:5])
