@@ -880,6 +880,234 @@ extern "C" int kappai_fixed_decay_chunks(const float* qf, const float* kf, const
 }
 
 // ---------------------------------------------------------------------------------------
+// A decay per token and key channel with the bonus for the own token, over long portions in
+// chunks of rows: o_i = (S_(i-1) + diag(u) k_i v_i^T)^T q_i, S_i = diag(a_i) S_(i-1) + k_i v_i^T.
+// With L_j = log a_0 + .. + log a_j inside the chunk (L_(-1) = 0) and S0 the state the chunk
+// starts from,
+//   o_i = sum_(j < i) [sum_r q_i[r] k_j[r] exp(L_(i-1)[r] - L_j[r])] v_j + (q_i . (u * k_i)) v_i
+//         + S0^T (q_i * exp(L_(i-1)))
+//   S   = diag(exp(L_(n-1))) S0 + sum_j (k_j * exp(L_(n-1) - L_j)) v_j^T.
+// Every exponent is a sum of logarithms of decays, so <= 0: nothing is ever divided by a decay.
+// The weights inside the brackets are made term by term on the vector units (an exponential a
+// term); everything else is the products of tiles of the fixed decay's kernels, and the same
+// three passes.  A decay that has underflowed to zero counts as exp(-200), which is zero again in
+// float32 while its logarithm stays finite.  `total` [n_chunks, H, d]: exp(L_(n-1)) of a chunk.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float fd_log_decay(float a) { return fmaxf(logf(a), -104.f); }
+
+template <typename TV>
+__global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_sums_kernel(
+    const float* __restrict__ kf, const float* __restrict__ af, const TV* __restrict__ v,
+    int v_stride, const int* __restrict__ chunks, int H, int d, int dv, int n_ct,
+    float* __restrict__ carry, float* __restrict__ total) {
+  __shared__ __attribute__((aligned(16))) float Ks[FD_C][FD_T];
+  __shared__ __attribute__((aligned(16))) float Vs[FD_C][FD_T];
+  __shared__ float Ls[FD_C][FD_T];
+  __shared__ float Ln[FD_T];
+  const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int ct = blockIdx.z % n_ct, c0 = ct * FD_T, r0 = (blockIdx.z / n_ct) * FD_T;
+  const int row0 = chunks[3 * ch + 1], n = min(chunks[3 * ch + 2], FD_C);
+  if (tid < FD_T) {
+    float run = 0.f;
+    const bool ok = r0 + tid < d;
+    for (int j = 0; j < n; ++j) {
+      if (ok) run += fd_log_decay(af[((size_t)(row0 + j) * H + h) * d + r0 + tid]);
+      Ls[j][tid] = run;
+    }
+    Ln[tid] = run;
+    if (ct == 0 && ok) total[((size_t)ch * H + h) * d + r0 + tid] = expf(run);
+  }
+  __syncthreads();
+  for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+    const int j = i / FD_T, e = i % FD_T;
+    const size_t row = (size_t)(row0 + j);
+    Ks[j][e] = (j < n && r0 + e < d)
+                   ? kf[(row * H + h) * d + r0 + e] * expf(fminf(Ln[e] - Ls[j][e], 0.f)) : 0.f;
+    Vs[j][e] = (j < n && c0 + e < dv) ? to_f32(v[row * v_stride + (size_t)h * dv + c0 + e]) : 0.f;
+  }
+  __syncthreads();
+  for (int tile = tid; tile < (FD_T / 4) * (FD_T / 4); tile += FD_THREADS) {
+    const int a0 = (tile / (FD_T / 4)) * 4, b0 = (tile % (FD_T / 4)) * 4;
+    float acc[4][4] = {};
+    fd_outer(acc, &Vs[0][0], FD_T, &Ks[0][0], FD_T, a0, b0, n);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int c = c0 + a0 + a, r = r0 + b0 + b;
+        if (c < dv && r < d) carry[(((size_t)ch * H + h) * dv + c) * d + r] = acc[a][b];
+      }
+  }
+}
+
+__global__ __launch_bounds__(256) void channel_decay_chunk_carry_kernel(
+    const float* __restrict__ total, const int* __restrict__ seg_chunk0,
+    const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot, int H, int d, int dv,
+    float* __restrict__ carry, float* __restrict__ state) {
+  const int seg = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x, n_el = dv * d;
+  if (e >= n_el) return;
+  const int ch0 = seg_chunk0[seg], ch1 = seg_chunk0[seg + 1];
+  if (ch0 >= ch1) return;
+  const int r = e % d;
+  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + e;
+  float S = seg_pos0[seg] > 0 ? *st : 0.f;
+  for (int c = ch0; c < ch1; c += 4) {
+    float own[4], fac[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int cc = min(c + i, ch1 - 1);
+      own[i] = carry[((size_t)cc * H + h) * n_el + e];
+      fac[i] = total[((size_t)cc * H + h) * d + r];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (c + i >= ch1) break;
+      carry[((size_t)(c + i) * H + h) * n_el + e] = S;      // the state the chunk starts from
+      S = fmaf(fac[i], S, own[i]);
+    }
+  }
+  *st = S;
+}
+
+template <typename TV>
+__global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_out_kernel(
+    const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ af,
+    const TV* __restrict__ v, int v_stride, const float* __restrict__ bonus,
+    const int* __restrict__ chunks, int H, int d, int dv, const float* __restrict__ carry,
+    float* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) float Qt[FD_T][FD_CS];     // [key channel][row]
+  __shared__ __attribute__((aligned(16))) float Kt[FD_T][FD_CS];
+  // Lx[r][0] = 0, Lx[r][j + 1] = L_j: row i reads L_(i-1) at [i], key row j its L_j at [j + 1]
+  __shared__ __attribute__((aligned(16))) float Lx[FD_T][FD_CS];
+  __shared__ __attribute__((aligned(16))) float Pt[FD_C][FD_CS];     // [key row j][query row i]
+  __shared__ __attribute__((aligned(16))) float Vs[FD_C][FD_T];      // [row][value channel]
+  __shared__ __attribute__((aligned(16))) float St[FD_T][FD_TS];     // [key channel][value channel]
+  const int ch = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * FD_T, tid = threadIdx.x;
+  const int row0 = chunks[3 * ch + 1], n = min(chunks[3 * ch + 2], FD_C);
+  // the weights of the chunk's own rows: 128 tiles of 4 rows i x 2 rows j
+  const int pi0 = (tid / (FD_C / 2)) * 4, pj0 = (tid % (FD_C / 2)) * 2;
+  const bool p_live = pj0 < pi0 + 3;            // (a tile with some j < i)
+  float accP[4][2] = {}, diag = 0.f;
+  // the outputs, 32 rows x 64 value channels: 128 tiles of 4 x 4
+  const int oi0 = (tid / (FD_T / 4)) * 4, oc0 = (tid % (FD_T / 4)) * 4;
+  float accO[4][4] = {}, accS[4][4] = {};
+  const float* S0 = carry + ((size_t)ch * H + h) * dv * d;
+  for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+    const int j = i / FD_T, e = i % FD_T;
+    Vs[j][e] = (j < n && c0 + e < dv)
+                   ? to_f32(v[(size_t)(row0 + j) * v_stride + (size_t)h * dv + c0 + e]) : 0.f;
+  }
+  for (int r0 = 0; r0 < d; r0 += FD_T) {
+    const int kn = min(FD_T, d - r0);
+    __syncthreads();
+    for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+      const int j = i / FD_T, e = i % FD_T;
+      const bool ok = j < n && r0 + e < d;
+      const size_t at = ((size_t)(row0 + j) * H + h) * d + r0 + e;
+      Qt[e][j] = ok ? qf[at] : 0.f;
+      Kt[e][j] = ok ? kf[at] : 0.f;
+    }
+    if (tid < FD_T) {
+      float run = 0.f;
+      Lx[tid][0] = 0.f;
+      const bool ok = r0 + tid < d;
+      for (int j = 0; j < FD_C; ++j) {
+        if (ok && j < n) run += fd_log_decay(af[((size_t)(row0 + j) * H + h) * d + r0 + tid]);
+        Lx[tid][j + 1] = run;
+      }
+    }
+    __syncthreads();
+    if (p_live) {
+      for (int r = 0; r < kn; ++r) {
+        const float4 q4 = *reinterpret_cast<const float4*>(&Qt[r][pi0]);
+        const float4 e4 = *reinterpret_cast<const float4*>(&Lx[r][pi0]);
+        const float q[4] = {q4.x, q4.y, q4.z, q4.w}, e[4] = {e4.x, e4.y, e4.z, e4.w};
+        const float k[2] = {Kt[r][pj0], Kt[r][pj0 + 1]};
+        const float l[2] = {Lx[r][pj0 + 1], Lx[r][pj0 + 2]};
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            accP[a][b] = fmaf(q[a] * k[b], __expf(fminf(e[a] - l[b], 0.f)), accP[a][b]);
+      }
+    }
+    if (tid < FD_C) {
+      const float* u = bonus + (size_t)h * d + r0;
+      for (int r = 0; r < kn; ++r) diag = fmaf(Qt[r][tid] * Kt[r][tid], u[r], diag);
+    }
+    __syncthreads();
+    for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
+      const int e = i / FD_C, j = i % FD_C;
+      Qt[e][j] *= expf(Lx[e][j]);
+    }
+    for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
+      const int c = i / FD_T, e = i % FD_T;
+      St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(c0 + c) * d + r0 + e] : 0.f;
+    }
+    __syncthreads();
+    fd_outer(accS, &Qt[0][0], FD_CS, &St[0][0], FD_TS, oi0, oc0, kn);
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int i = pi0 + a, j = pj0 + b;
+      Pt[j][i] = (j < i && i < n) ? accP[a][b] : 0.f;
+    }
+  __syncthreads();
+  if (tid < FD_C) Pt[tid][tid] = tid < n ? diag : 0.f;
+  __syncthreads();
+  fd_outer(accO, &Pt[0][0], FD_CS, &Vs[0][0], FD_T, oi0, oc0, n);
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int i = oi0 + a;
+    if (i >= n) continue;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int c = c0 + oc0 + b;
+      if (c < dv) out[((size_t)(row0 + i) * H + h) * dv + c] = accO[a][b] + accS[a][b];
+    }
+  }
+}
+
+// As kappai_fixed_decay_chunks, with af [T, H, d] the decays as recurrence_prep leaves them,
+// bonus [H, d], and total [n_chunks, H, d] floats of scratch beside carry.
+extern "C" int kappai_channel_decay_chunks(const float* qf, const float* kf, const float* af,
+                                           const void* v, int v_stride, int v_is_bf16,
+                                           const float* bonus, float* state, const int* seg_pos0,
+                                           const int* seg_slot, const int* chunks,
+                                           const int* seg_chunk0, int n_chunks, int chunk_rows,
+                                           int T, int S, int H, int d, int dv, float* carry,
+                                           float* total, float* out, hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (H < 1 || H > 65535 || d < 1 || dv < 1 || n_chunks < 1 || chunk_rows < 1 ||
+      chunk_rows > FD_C || !chunks || !seg_chunk0 || !carry || !total || !bonus || !af)
+    return (int)hipErrorInvalidValue;
+  const int n_ct = (dv + FD_T - 1) / FD_T, n_rt = (d + FD_T - 1) / FD_T;
+  const int el_blocks = (dv * d + 255) / 256;
+  if (n_ct * n_rt > 65535 || el_blocks > 65535) return (int)hipErrorInvalidValue;
+  const dim3 sums(n_chunks, H, n_ct * n_rt), outs(n_chunks, H, n_ct);
+  if (v_is_bf16)
+    hipLaunchKernelGGL(channel_decay_chunk_sums_kernel<bf16_t>, sums, dim3(FD_THREADS), 0, stream,
+                       kf, af, (const bf16_t*)v, v_stride, chunks, H, d, dv, n_ct, carry, total);
+  else
+    hipLaunchKernelGGL(channel_decay_chunk_sums_kernel<float>, sums, dim3(FD_THREADS), 0, stream,
+                       kf, af, (const float*)v, v_stride, chunks, H, d, dv, n_ct, carry, total);
+  hipLaunchKernelGGL(channel_decay_chunk_carry_kernel, dim3(S, H, el_blocks), dim3(256), 0,
+                     stream, total, seg_chunk0, seg_pos0, seg_slot, H, d, dv, carry, state);
+  if (v_is_bf16)
+    hipLaunchKernelGGL(channel_decay_chunk_out_kernel<bf16_t>, outs, dim3(FD_THREADS), 0, stream,
+                       qf, kf, af, (const bf16_t*)v, v_stride, bonus, chunks, H, d, dv, carry,
+                       out);
+  else
+    hipLaunchKernelGGL(channel_decay_chunk_out_kernel<float>, outs, dim3(FD_THREADS), 0, stream,
+                       qf, kf, af, (const float*)v, v_stride, bonus, chunks, H, d, dv, carry,
+                       out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // Per head: o / sqrt(mean(o^2) + eps) * weight[dv] * gate, gate = silu(g) (kind 0) or sigmoid(g)
 // (kind 1) of the projection g [T, >= H dv] with a row stride.  A wave a (row, head).
 // weight_stride: 0 when the heads share one weight [dv], dv when each has its own [H, dv].

@@ -2034,8 +2034,9 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     token from global memory, or a block of waves that takes the tokens in chunks through LDS.
 
     ``chunks`` [n, 3] = (segment, first row, rows <= ``chunk_rows`` <= 32) with ``seg_chunk0``
-    [S + 1], as for ``mingru_scan``: a fixed decay (no ``beta``, no ``bonus``, H == Hk) is then
-    worked chunk by chunk in three passes, with no chain along the tokens of a chunk."""
+    [S + 1], as for ``mingru_scan``: a fixed decay (no ``beta``, no ``bonus``, H == Hk) and the
+    form with a ``bonus`` are then worked chunk by chunk in three passes, with no chain along the
+    tokens of a chunk (every factor is a product of decays, none is divided by one)."""
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     _need(form in SCAN_FORMS, lambda: f"matrix_state_recurrence: form {form!r}")
     _need(decay in DECAY_KINDS and (z is None) == (decay == "fixed")
@@ -2091,7 +2092,7 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     out = torch.empty((T, H * dv), dtype=F32, device=dev)
     values = vf if silu_inputs else v
     mode = 1 if beta is not None else 2 if bonus is not None else 0
-    if chunks is not None and decay == "fixed" and mode == 0 and H == Hk:
+    if chunks is not None and H == Hk and ((decay == "fixed" and mode == 0) or mode == 2):
         _gpu("chunks", chunks, I32)
         _gpu("seg_chunk0", seg_chunk0, I32)
         _need(chunks.dim() == 2 and chunks.shape[1] == 3 and seg_chunk0.shape[0] == S + 1
@@ -2100,6 +2101,15 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       f"{chunk_rows} rows do not fit")
         n_chunks = chunks.shape[0]
         carry = torch.empty((n_chunks, H, dv, d), dtype=F32, device=dev)
+        if mode == 2:
+            total = torch.empty((n_chunks, H, d), dtype=F32, device=dev)
+            check(lib.kappai_channel_decay_chunks(
+                _ptr(qf), _ptr(kf), _ptr(af), _ptr(values), _c_int(values.stride(0)),
+                _c_int(_is_bf16(values.dtype)), _ptr(bonus), _ptr(state), _ptr(seg_pos0),
+                _ptr(seg_slot), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks),
+                _c_int(chunk_rows), _c_int(T), _c_int(S), _c_int(H), _c_int(d), _c_int(dv),
+                _ptr(carry), _ptr(total), _ptr(out), _stream()), "channel_decay_chunks")
+            return out
         check(lib.kappai_fixed_decay_chunks(
             _ptr(qf), _ptr(kf), _ptr(values), _c_int(values.stride(0)),
             _c_int(_is_bf16(values.dtype)), _ptr(rate), _ptr(state), _ptr(seg_pos0),

@@ -209,6 +209,10 @@ class BonusTimeMixing(Mixer):
     def _linears(self):
         return (self.r, self.k, self.v, self.g, self.w1, self.w2, self.out)
 
+    @property
+    def step_tables(self) -> ScanChunks:
+        return ScanChunks(min(tuning.SCAN_CHUNK_ROWS, ops.FIXED_DECAY_CHUNK_ROWS))
+
     def cache_spec(self):
         return CacheBundle((("state", FixedState((self.H, self.d, self.d), "float32")),
                             ("shift", FixedState((self.width,), "float32"))))
@@ -241,11 +245,16 @@ class BonusTimeMixing(Mixer):
         with profile.scope("ffn_act"):
             low = ops.tanh(self.w1.forward(mixes[4]))
         z = self.w2.forward(low)
+        # long portions: chunk by chunk (the factors between two tokens are products of decays)
+        chunked = batch.max_segment_rows > tuning.SCAN_CHUNKS_FROM_ROWS
         with profile.scope("scan"):
             o = ops.matrix_state_recurrence(
                 r, k, v, z, H, H, d, d, None, self.w0, 1.0, 1.0, cache.part("state").state,
                 batch.seg_start, batch.seg_pos0, batch.seg_slot, decay="double_exp",
-                bonus=self.bonus)
+                bonus=self.bonus,
+                chunks=batch.extra.get("scan_chunks") if chunked else None,
+                seg_chunk0=batch.extra.get("scan_seg_chunk0") if chunked else None,
+                chunk_rows=min(tuning.SCAN_CHUNK_ROWS, ops.FIXED_DECAY_CHUNK_ROWS))
             y = ops.head_norm_gate(o, self.norm_w, self.norm_eps, g, ops.GATE_SILU, H, d,
                                    self.dtype)
         return self.out.forward(y, partial_sums=True)

@@ -247,20 +247,35 @@ def chunk_tables(segments, rows):
 @pytest.mark.parametrize("H,d,dv", [(3, 8, 16), (1, 72, 24), (2, 136, 8), (2, 24, 70),
                                     (2, 64, 128), (1, 300, 4), (5, 20, 20), (2, 64, 200)])
 @pytest.mark.parametrize("rows", [32, 7])
-def test_a_fixed_decay_chunk_by_chunk(H, d, dv, rows):
+@pytest.mark.parametrize("kind", ["fixed", "bonus"])
+def test_recurrences_chunk_by_chunk(H, d, dv, rows, kind):
     """Three unequal requests side by side, in portions that end inside a chunk and single rows
-    (slots in another order, NaN in the states before), by the form that works chunks of rows in
-    passes: against a loop in float64, and against the kernel that walks the tokens."""
+    (slots in another order, NaN in the states before), by the forms that work chunks of rows in
+    passes: against a loop in float64, and against the kernel that walks the tokens.  The decays
+    of the form with a bonus reach from next to one down to nothing at all (a decay that
+    underflows to zero: what came before is gone)."""
     from kappai_amd.kernels import ops
+    if kind == "bonus":
+        dv = d
     g = gen(12)
     lens = [150, 77, 120]
     seqs = [dict(q=torch.randn(n, H * d, generator=g) * 0.5, k=torch.randn(n, H * d, generator=g),
-                 v=torch.randn(n, H * dv, generator=g)) for n in lens]
+                 v=torch.randn(n, H * dv, generator=g),
+                 z=torch.randn(n, H * d, generator=g) * 2.5 - 2.0) for n in lens]
+    seqs[0]["z"][40, :d // 2 + 1] = 6.0           # exp(-exp(6)) is zero in float32
     rate = torch.tensor(([1.0, 0.0, 0.9, 0.5, 0.97] * 2)[:H])
+    w0 = torch.randn(H * d, generator=g) * 0.5
+    bonus = torch.randn(H, d, generator=g)
     want = []
     for s, n in zip(seqs, lens):
-        q, k, v = (P.silu(s[c].double()).reshape(n, H, -1) for c in "qkv")
-        want.append(plain_state_scan(q, k, v, rate.double()[None, :, None].expand(n, H, d), None))
+        if kind == "fixed":
+            q, k, v = (P.silu(s[c].double()).reshape(n, H, -1) for c in "qkv")
+            want.append(plain_state_scan(q, k, v, rate.double()[None, :, None].expand(n, H, d),
+                                         None))
+        else:
+            q, k, v = (s[c].double().reshape(n, H, -1) for c in "qkv")
+            a = torch.exp(-torch.exp(s["z"].double() + w0.double())).reshape(n, H, d)
+            want.append(plain_state_scan(q, k, v, a, bonus.double()))
     states = [torch.full((6, H, dv, d), float("nan"), device=DEV) for _ in range(2)]
     got, walked, done = [[], [], []], [[], [], []], [0, 0, 0]
     for step in ([70, 33, 1], [1, 1, 64], [40, 43, 2], [39, 0, 53]):
@@ -269,14 +284,20 @@ def test_a_fixed_decay_chunk_by_chunk(H, d, dv, rows):
         tb = tables(segs, slots=[[4, 0, 2][i] for i in live])
         ch, first = chunk_tables(segs, rows)
         cat = {c: torch.cat([seqs[i][c][done[i]:done[i] + step[i]] for i in live]).to(DEV)
-               for c in "qkv"}
+               for c in "qkvz"}
         outs = []
         for st, kw in ((states[0], dict(chunks=ch, seg_chunk0=first, chunk_rows=rows)),
                        (states[1], {})):
-            outs.append(ops.matrix_state_recurrence(
-                cat["q"], cat["k"], cat["v"], None, H, H, d, dv, rate.to(DEV), None, 1.0, 1.0,
-                st, tb["seg_start"], tb["seg_pos0"], tb["seg_slot"], decay="fixed",
-                silu_inputs=True, **kw))
+            if kind == "fixed":
+                outs.append(ops.matrix_state_recurrence(
+                    cat["q"], cat["k"], cat["v"], None, H, H, d, dv, rate.to(DEV), None, 1.0, 1.0,
+                    st, tb["seg_start"], tb["seg_pos0"], tb["seg_slot"], decay="fixed",
+                    silu_inputs=True, **kw))
+            else:
+                outs.append(ops.matrix_state_recurrence(
+                    cat["q"], cat["k"], cat["v"], cat["z"], H, H, d, dv, None, w0.to(DEV), 1.0,
+                    1.0, st, tb["seg_start"], tb["seg_pos0"], tb["seg_slot"], decay="double_exp",
+                    bonus=bonus.to(DEV), **kw))
         at = 0
         for i in live:
             got[i].append(outs[0][at:at + step[i]])
@@ -481,10 +502,14 @@ def test_bonus_time_mixing_part(dtype, tol, H, d, rank):
     t = bind_random(part, 9, dtype)
     cm = CacheManager([part.cache_spec()], 16, 1, 2)
     cm.allocate_storage(dtype, DEV, poison=True)
-    x = torch.randn(150, 72, generator=gen(18)).to(BF16)
-    got, _ = step_through(part, cm, x.to(dtype), PORTIONS_150, cm.view(0))
     m = {"heads": H, "dim": d}
-    assert rel(got, P.bonus_time_mixing(x.double(), t, "a.", m, 1e-5)) < tol
+    # short portions and single tokens; then portions long enough to be worked chunk by chunk
+    for T, portions, seed in ((150, PORTIONS_150, 18), (330, [200, 1, 97, 2, 30], 27)):
+        cm = CacheManager([part.cache_spec()], 16, 1, 2)
+        cm.allocate_storage(dtype, DEV, poison=True)
+        x = torch.randn(T, 72, generator=gen(seed)).to(BF16)
+        got, _ = step_through(part, cm, x.to(dtype), portions, cm.view(0))
+        assert rel(got, P.bonus_time_mixing(x.double(), t, "a.", m, 1e-5)) < tol, T
 
 
 def test_the_bonus_weighs_the_token_itself_and_the_shift_reads_the_token_before():
