@@ -681,7 +681,8 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
 // from; the chunks' outputs side by side.  Everything is float32 on the vector units (scores,
 // their weights and the state are asked for in 32 bits): products of tiles staged in LDS so that
 // the summed index is the row of both operands, a thread keeping 4 x 4 results.
-// `carry` [n_chunks, H, dv, d] (a head's matrix column by column, as the state).
+// `carry` [n_chunks, H, d, dv] (a head's matrix row by row: a row of S0 is one stretch for the
+// pass that multiplies by it; the state itself lies column by column).
 // ---------------------------------------------------------------------------------------
 #define FD_C 32         // most rows of a chunk
 #define FD_T 64         // key channels / value channels a tile
@@ -689,9 +690,16 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
 #define FD_CS (FD_C + 4)   // row strides in LDS: multiples of four floats, off the powers of two
 #define FD_TS (FD_T + 4)
 
+// Element i of a tile of FD_C rows x FD_T channels that is read from rows of channels and stored
+// [channel][row]: a wave's lanes take eight channels of eight rows, so that their stores fall on
+// all the banks (a row stride of FD_CS floats puts neighbouring channels four banks apart).
+__device__ __forceinline__ int fd_spread_e(int i) { return (i % 8) + 8 * ((i / 64) % (FD_T / 8)); }
+__device__ __forceinline__ int fd_spread_j(int i) { return ((i / 8) % 8) + 8 * (i / (8 * FD_T)); }
+
 // acc[a][b] += sum_(k < kn) X[k][a0 + a] * Y[k][b0 + b]
 __device__ __forceinline__ void fd_outer(float (&acc)[4][4], const float* X, int xs, const float* Y,
                                          int ys, int a0, int b0, int kn) {
+#pragma unroll 4
   for (int k = 0; k < kn; ++k) {
     const float4 x4 = *reinterpret_cast<const float4*>(X + k * xs + a0);
     const float4 y4 = *reinterpret_cast<const float4*>(Y + k * ys + b0);
@@ -732,7 +740,7 @@ __global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_sums_kernel(
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const int c = c0 + a0 + a, r = r0 + b0 + b;
-        if (c < dv && r < d) carry[(((size_t)ch * H + h) * dv + c) * d + r] = acc[a][b];
+        if (c < dv && r < d) carry[(((size_t)ch * H + h) * d + r) * dv + c] = acc[a][b];
       }
   }
 }
@@ -748,7 +756,7 @@ __global__ __launch_bounds__(256) void fixed_decay_chunk_carry_kernel(
   const int ch0 = seg_chunk0[seg], ch1 = seg_chunk0[seg + 1];
   if (ch0 >= ch1) return;
   const float lam = rate[h], lam_full = powf(lam, (float)FD_C);
-  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + e;
+  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + (size_t)(e % dv) * d + e / dv;
   float S = seg_pos0[seg] > 0 ? *st : 0.f;
   for (int c = ch0; c < ch1; c += 4) {
     float own[4];
@@ -789,7 +797,7 @@ __global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_out_kernel(
   for (int r0 = 0; r0 < d; r0 += FD_T) {
     __syncthreads();
     for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
-      const int j = i / FD_T, e = i % FD_T;
+      const int e = fd_spread_e(i), j = fd_spread_j(i);
       const bool ok = j < n && r0 + e < d;
       const size_t at = ((size_t)(row0 + j) * H + h) * d + r0 + e;
       Qt[e][j] = ok ? qf[at] : 0.f;
@@ -822,12 +830,22 @@ __global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_out_kernel(
   for (int r0 = 0; r0 < d; r0 += FD_T) {
     __syncthreads();
     for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
-      const int j = i / FD_T, e = i % FD_T;
+      const int e = fd_spread_e(i), j = fd_spread_j(i);
       Qt[e][j] = (j < n && r0 + e < d) ? qf[((size_t)(row0 + j) * H + h) * d + r0 + e] : 0.f;
     }
-    for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
-      const int c = i / FD_T, e = i % FD_T;
-      St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(c0 + c) * d + r0 + e] : 0.f;
+    if (dv % 4 == 0) {
+      for (int i = tid; i < FD_T * FD_T / 4; i += FD_THREADS) {
+        const int e = i / (FD_T / 4), c = (i % (FD_T / 4)) * 4;
+        float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c0 + c < dv && r0 + e < d)
+          s4 = *reinterpret_cast<const float4*>(S0 + (size_t)(r0 + e) * dv + c0 + c);
+        *reinterpret_cast<float4*>(&St[e][c]) = s4;
+      }
+    } else {
+      for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
+        const int e = i / FD_T, c = i % FD_T;
+        St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(r0 + e) * dv + c0 + c] : 0.f;
+      }
     }
     __syncthreads();
     fd_outer(accS, &Qt[0][0], FD_CS, &St[0][0], FD_TS, oi0, oc0, min(FD_T, d - r0));
@@ -847,7 +865,7 @@ __global__ __launch_bounds__(FD_THREADS) void fixed_decay_chunk_out_kernel(
 
 // qf, kf [T, H, d] float32 as recurrence_prep leaves them, v [T, >= H dv] with a row stride,
 // rate [H] the decays, chunks [n_chunks, 3] = (segment, first row, rows <= 32), seg_chunk0
-// [S + 1], carry [n_chunks, H, dv, d] floats of scratch, state [slots, H, dv, d], out [T, H dv].
+// [S + 1], carry [n_chunks, H, d, dv] floats of scratch, state [slots, H, dv, d], out [T, H dv].
 extern "C" int kappai_fixed_decay_chunks(const float* qf, const float* kf, const void* v,
                                          int v_stride, int v_is_bf16, const float* rate,
                                          float* state, const int* seg_pos0, const int* seg_slot,
@@ -935,7 +953,7 @@ __global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_sums_kernel(
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const int c = c0 + a0 + a, r = r0 + b0 + b;
-        if (c < dv && r < d) carry[(((size_t)ch * H + h) * dv + c) * d + r] = acc[a][b];
+        if (c < dv && r < d) carry[(((size_t)ch * H + h) * d + r) * dv + c] = acc[a][b];
       }
   }
 }
@@ -949,8 +967,8 @@ __global__ __launch_bounds__(256) void channel_decay_chunk_carry_kernel(
   if (e >= n_el) return;
   const int ch0 = seg_chunk0[seg], ch1 = seg_chunk0[seg + 1];
   if (ch0 >= ch1) return;
-  const int r = e % d;
-  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + e;
+  const int r = e / dv;
+  float* st = state + ((size_t)seg_slot[seg] * H + h) * n_el + (size_t)(e % dv) * d + r;
   float S = seg_pos0[seg] > 0 ? *st : 0.f;
   for (int c = ch0; c < ch1; c += 4) {
     float own[4], fac[4];
@@ -1002,7 +1020,7 @@ __global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_out_kernel(
     const int kn = min(FD_T, d - r0);
     __syncthreads();
     for (int i = tid; i < FD_C * FD_T; i += FD_THREADS) {
-      const int j = i / FD_T, e = i % FD_T;
+      const int e = fd_spread_e(i), j = fd_spread_j(i);
       const bool ok = j < n && r0 + e < d;
       const size_t at = ((size_t)(row0 + j) * H + h) * d + r0 + e;
       Qt[e][j] = ok ? qf[at] : 0.f;
@@ -1019,6 +1037,7 @@ __global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_out_kernel(
     }
     __syncthreads();
     if (p_live) {
+#pragma unroll 2
       for (int r = 0; r < kn; ++r) {
         const float4 q4 = *reinterpret_cast<const float4*>(&Qt[r][pi0]);
         const float4 e4 = *reinterpret_cast<const float4*>(&Lx[r][pi0]);
@@ -1041,9 +1060,19 @@ __global__ __launch_bounds__(FD_THREADS) void channel_decay_chunk_out_kernel(
       const int e = i / FD_C, j = i % FD_C;
       Qt[e][j] *= expf(Lx[e][j]);
     }
-    for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
-      const int c = i / FD_T, e = i % FD_T;
-      St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(c0 + c) * d + r0 + e] : 0.f;
+    if (dv % 4 == 0) {
+      for (int i = tid; i < FD_T * FD_T / 4; i += FD_THREADS) {
+        const int e = i / (FD_T / 4), c = (i % (FD_T / 4)) * 4;
+        float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c0 + c < dv && r0 + e < d)
+          s4 = *reinterpret_cast<const float4*>(S0 + (size_t)(r0 + e) * dv + c0 + c);
+        *reinterpret_cast<float4*>(&St[e][c]) = s4;
+      }
+    } else {
+      for (int i = tid; i < FD_T * FD_T; i += FD_THREADS) {
+        const int e = i / FD_T, c = i % FD_T;
+        St[e][c] = (c0 + c < dv && r0 + e < d) ? S0[(size_t)(r0 + e) * dv + c0 + c] : 0.f;
+      }
     }
     __syncthreads();
     fd_outer(accS, &Qt[0][0], FD_CS, &St[0][0], FD_TS, oi0, oc0, kn);
@@ -1112,19 +1141,29 @@ extern "C" int kappai_channel_decay_chunks(const float* qf, const float* kf, con
 // (kind 1) of the projection g [T, >= H dv] with a row stride.  A wave a (row, head).
 // weight_stride: 0 when the heads share one weight [dv], dv when each has its own [H, dv].
 // ---------------------------------------------------------------------------------------
+#define HNG_WIDE_THREADS 256      // heads of more than 512 values take a block of four waves
 template <typename T>
-__global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(
+__global__ __launch_bounds__(HNG_WIDE_THREADS) void head_norm_gate_kernel(
     const float* __restrict__ o, const float* __restrict__ weight, float eps,
     const T* __restrict__ g, int g_stride, int gate_kind, int H, int dv, int weight_stride,
     T* __restrict__ out) {
+  __shared__ float part[HNG_WIDE_THREADS / WAVE];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int threads = blockDim.x;
   weight += (size_t)h * weight_stride;
   const float* orow = o + ((size_t)t * H + h) * dv;
   float ss = 0.f;
-  for (int e = lane; e < dv; e += WAVE) ss = fmaf(orow[e], orow[e], ss);
-  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+  for (int e = lane; e < dv; e += threads) ss = fmaf(orow[e], orow[e], ss);
+  ss = wave_sum(ss);
+  if (threads > WAVE) {
+    if (lane % WAVE == 0) part[lane / WAVE] = ss;
+    __syncthreads();
+    ss = 0.f;
+    for (int w = 0; w < threads / WAVE; ++w) ss += part[w];
+  }
+  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
   const T* gr = g + (size_t)t * g_stride + (size_t)h * dv;
-  for (int e = lane; e < dv; e += WAVE) {
+  for (int e = lane; e < dv; e += threads) {
     const float gv = to_f32(gr[e]);
     const float gate = gate_kind == 0 ? gv * la_sigmoid(gv) : la_sigmoid(gv);
     from_f32(out + ((size_t)t * H + h) * dv + e, orow[e] * inv * weight[e] * gate);
@@ -1138,11 +1177,12 @@ extern "C" int kappai_head_norm_gate(const float* o, const float* weight, float 
   if (T <= 0) return 0;
   if (H < 1 || H > 65535 || dv < 1 || gate_kind < 0 || gate_kind > 1)
     return (int)hipErrorInvalidValue;
+  const dim3 block(dv > 512 ? HNG_WIDE_THREADS : WAVE);
   if (is_bf16)
-    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(T, H), dim3(WAVE), 0, stream, o, weight,
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(T, H), block, 0, stream, o, weight,
                        eps, (const bf16_t*)g, g_stride, gate_kind, H, dv, weight_stride, (bf16_t*)out);
   else
-    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(T, H), dim3(WAVE), 0, stream, o, weight,
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(T, H), block, 0, stream, o, weight,
                        eps, (const float*)g, g_stride, gate_kind, H, dv, weight_stride, (float*)out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
