@@ -28,12 +28,14 @@ __device__ __forceinline__ void mingru_gates(float pz, float pu, float& a, float
 template <typename TP>
 struct scan_in {
   const TP* proj;          // KIND 0: [T, 3W]; KIND 1: the gated branch, rows `y_stride` apart
-  const float* gates;      // KIND 1: [T, 2W]
-  const float* gate_bias;  // KIND 1: [2W], added to the gates before their sigmoid
+  const float* gates;      // KIND 1: [T, 2W]: (r | i) for all channels, or with `gate_part` > 0
+                           // block by block, (r | i) of `gate_part` channels each
+  const float* gate_bias;  // KIND 1: [2W] laid out as a row of gates, added before their sigmoid
   const TP* u;             // KIND 1: [T, W]
   const float* sp;         // KIND 1: [W]
   float rate;              // KIND 1
   int y_stride;            // KIND 1
+  int gate_part;           // KIND 1: channels a block of the gates' layout (0: no blocks)
 };
 
 // a, b of row t and channel c, and (OUT) the factor on the state that makes the output
@@ -48,12 +50,14 @@ __device__ __forceinline__ void scan_terms(const scan_in<TP>& in, int W, int t, 
       g = pg * sigmoid_f(pg);
     }
   } else {
-    const float* gp = in.gates + (size_t)t * 2 * W + c;
+    const int part = in.gate_part;
+    const int at_r = part ? (c / part) * 2 * part + c % part : c, at_i = at_r + (part ? part : W);
+    const float* gp = in.gates + (size_t)t * 2 * W;
     const float uu = to_f32(in.u[(size_t)t * W + c]);
     // (1 - a^2 from the logarithm: a decay close to one loses nothing to cancellation)
-    const float la = -in.rate * sigmoid_f(gp[0] + in.gate_bias[c]) * in.sp[c];
+    const float la = -in.rate * sigmoid_f(gp[at_r] + in.gate_bias[at_r]) * in.sp[c];
     a = expf(la);
-    b = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f)) * sigmoid_f(gp[W] + in.gate_bias[W + c]) * uu;
+    b = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f)) * sigmoid_f(gp[at_i] + in.gate_bias[at_i]) * uu;
     if (OUT) {
       const float z = to_f32(in.proj[(size_t)t * in.y_stride + c]);
       g = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
@@ -203,17 +207,17 @@ extern "C" int kappai_mingru_scan(const void* proj, int proj_is_bf16, float* sta
   if (proj_is_bf16 && !out_is_bf16) return (int)hipErrorInvalidValue;
   if (proj_is_bf16)
     scan_launch<0, bf16_t, bf16_t>(scan_in<bf16_t>{(const bf16_t*)proj, nullptr, nullptr, nullptr, nullptr,
-                                                   0.f, 0},
+                                                   0.f, 0, 0},
                                    state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
                                    n_chunks, carry, out, stream);
   else if (out_is_bf16)
     scan_launch<0, float, bf16_t>(scan_in<float>{(const float*)proj, nullptr, nullptr, nullptr, nullptr,
-                                                 0.f, 0},
+                                                 0.f, 0, 0},
                                   state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
                                   n_chunks, carry, out, stream);
   else
     scan_launch<0, float, float>(scan_in<float>{(const float*)proj, nullptr, nullptr, nullptr, nullptr,
-                                                0.f, 0},
+                                                0.f, 0, 0},
                                  state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
                                  n_chunks, carry, out, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
@@ -222,24 +226,26 @@ extern "C" int kappai_mingru_scan(const void* proj, int proj_is_bf16, float* sta
 // The real-gated unit through the same kernels; `out` is stored as `u` and `y` are.
 extern "C" int kappai_gated_unit_scan(const float* gates, const float* gate_bias, const void* u,
                                       const void* y,
-                                      int y_stride, const float* sp, float rate, int is_bf16,
+                                      int y_stride, const float* sp, float rate, int gate_part,
+                                      int is_bf16,
                                       float* state, const int* seg_start, const int* seg_pos0,
                                       const int* seg_slot, int T, int S, int W, const int* chunks,
                                       const int* seg_chunk0, int n_chunks, float* carry, void* out,
                                       hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
-  if (S > 65535 || n_chunks > 65535 || W < 1 || y_stride < W || gate_bias == nullptr)
+  if (S > 65535 || n_chunks > 65535 || W < 1 || y_stride < W || gate_bias == nullptr ||
+      gate_part < 0 || (gate_part && W % gate_part))
     return (int)hipErrorInvalidValue;
   if (chunks != nullptr && (n_chunks <= 0 || carry == nullptr || seg_chunk0 == nullptr))
     return (int)hipErrorInvalidValue;
   if (is_bf16)
     scan_launch<1, bf16_t, bf16_t>(scan_in<bf16_t>{(const bf16_t*)y, gates, gate_bias, (const bf16_t*)u, sp,
-                                                   rate, y_stride},
+                                                   rate, y_stride, gate_part},
                                    state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
                                    n_chunks, carry, out, stream);
   else
     scan_launch<1, float, float>(scan_in<float>{(const float*)y, gates, gate_bias, (const float*)u, sp, rate,
-                                                y_stride},
+                                                y_stride, gate_part},
                                  state, seg_start, seg_pos0, seg_slot, S, W, chunks, seg_chunk0,
                                  n_chunks, carry, out, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();

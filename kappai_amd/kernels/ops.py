@@ -1417,12 +1417,14 @@ def gated_unit_scan(gates: torch.Tensor, gate_bias: torch.Tensor, u: torch.Tenso
                     rate: float, state: torch.Tensor, seg_start: torch.Tensor,
                     seg_pos0: torch.Tensor, seg_slot: torch.Tensor,
                     chunks: Optional[torch.Tensor] = None,
-                    seg_chunk0: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    seg_chunk0: Optional[torch.Tensor] = None, gate_part: int = 0) -> torch.Tensor:
     """The real-gated linear unit per channel: ``a = exp(-rate * sigmoid(g_r) * softplus_lam)``,
     ``S = a S + sqrt(1 - a^2) * sigmoid(g_i) * u``, output ``S * gelu_tanh(y)``.  ``gates``
     [T, 2W] float32 = (g_r | g_i) before the sigmoid and without ``gate_bias`` [2W], ``u`` [T, W], ``y`` [T, >= W] (a view with a
     row stride) as a product stored them, ``softplus_lam`` [W] float32, ``state`` [slots, W]
-    float32.  ``chunks`` / ``seg_chunk0`` as for ``mingru_scan``.  Returns [T, W] as ``u`` is
+    float32.  ``gate_part`` > 0: ``gates`` and ``gate_bias`` are laid out block by block, (g_r | g_i)
+    of ``gate_part`` channels each (what one product a block leaves), not (g_r | g_i) of all
+    channels.  ``chunks`` / ``seg_chunk0`` as for ``mingru_scan``.  Returns [T, W] as ``u`` is
     stored."""
     _gpu("gates", gates, F32)
     _gpu("gate_bias", gate_bias, F32)
@@ -1433,7 +1435,8 @@ def gated_unit_scan(gates: torch.Tensor, gate_bias: torch.Tensor, u: torch.Tenso
     T, W = u.shape
     _need(tuple(gates.shape) == (T, 2 * W) and gate_bias.shape == (2 * W,) and y.dim() == 2 and y.shape[0] == T
           and y.shape[1] >= W and y.stride(1) == 1 and softplus_lam.shape == (W,)
-          and state.dim() == 2 and state.shape[1] == W,
+          and state.dim() == 2 and state.shape[1] == W
+          and gate_part >= 0 and (gate_part == 0 or W % gate_part == 0),
           lambda: f"gated_unit_scan: gates {tuple(gates.shape)}, u {tuple(u.shape)}, y "
                   f"{tuple(y.shape)}, state {tuple(state.shape)}")
     for name, t in (("seg_start", seg_start), ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
@@ -1452,7 +1455,7 @@ def gated_unit_scan(gates: torch.Tensor, gate_bias: torch.Tensor, u: torch.Tenso
         carry = torch.empty((n_chunks, 3, W), dtype=F32, device=u.device)
     check(library("mingru").kappai_gated_unit_scan(
         _ptr(gates), _ptr(gate_bias), _ptr(u), _ptr(y), _c_int(y.stride(0)), _ptr(softplus_lam),
-        _c_float(rate),
+        _c_float(rate), _c_int(gate_part),
         _c_int(_is_bf16(u.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot),
         _c_int(T), _c_int(S), _c_int(W), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks),
         _ptr(carry), _ptr(out), _stream()), "gated_unit_scan")

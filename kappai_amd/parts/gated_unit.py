@@ -80,8 +80,10 @@ class RealGatedUnit(Mixer):
         self.conv_taps = tensors[self._conv].to(torch.float32).contiguous()
         self.conv_bias = tensors[self._conv_bias].to(torch.float32).contiguous()
         (wr, br), (wi, bi) = ((tensors[w], tensors[b]) for w, b in self._gates)
-        self.gate_w = (wr.contiguous(), wi.contiguous())        # each [blocks, part, part]
-        self.gate_b = torch.cat([br.reshape(-1), bi.reshape(-1)]).to(torch.float32).contiguous()
+        # both gates of a block from one product: [blocks, r | i, part], biases laid out alike
+        self.gate_w = torch.cat([wr, wi], dim=1).contiguous()
+        self.gate_b = torch.cat([br.reshape(self.blocks, -1), bi.reshape(self.blocks, -1)],
+                                dim=1).reshape(-1).to(torch.float32).contiguous()
         lam = tensors[self._lam].to(torch.float64)
         self.softplus_lam = torch.nn.functional.softplus(lam).to(torch.float32).contiguous()
 
@@ -102,22 +104,22 @@ class RealGatedUnit(Mixer):
                               bias=self.conv_bias, activation=False)
         chunked = batch.max_segment_rows > tuning.SCAN_CHUNKS_FROM_ROWS
         with profile.scope("scan"):
-            # (r | i) before their sigmoid, float32 sums: a matrix a part of the channels
+            # (r | i) of every block before their sigmoid, float32 sums: a matrix a block
             gates = torch.empty((u.shape[0], 2 * C), dtype=torch.float32, device=u.device)
             part = C // self.blocks
-            for side, w in enumerate(self.gate_w):
-                ops.headwise_linear(u, part, w, out=gates[:, side * C:(side + 1) * C],
-                                    out_head_stride=part, out_dtype=torch.float32)
+            ops.headwise_linear(u, part, self.gate_w, out=gates, out_head_stride=2 * part,
+                                out_dtype=torch.float32)
             y = ops.gated_unit_scan(
-                gates, self.gate_b, u, proj[:, C:], self.softplus_lam, self.rate, state, batch.seg_start,
-                batch.seg_pos0, batch.seg_slot,
+                gates, self.gate_b, u, proj[:, C:], self.softplus_lam, self.rate, state,
+                batch.seg_start, batch.seg_pos0, batch.seg_slot,
                 chunks=batch.extra.get("scan_chunks") if chunked else None,
-                seg_chunk0=batch.extra.get("scan_seg_chunk0") if chunked else None)
+                seg_chunk0=batch.extra.get("scan_seg_chunk0") if chunked else None,
+                gate_part=part)
         return self.out.forward(y, partial_sums=True)
 
     def weight_bytes(self) -> int:
         return (self.inputs.weight_bytes() + self.out.weight_bytes()
-                + sum(w.numel() * w.element_size() for w in self.gate_w))
+                + self.gate_w.numel() * self.gate_w.element_size())
 
 
 register_part("mixer", "real_gated_unit", RealGatedUnit)

@@ -615,9 +615,11 @@ def tanh(x):
 
 
 def gated_unit_scan(gates, gate_bias, u, y, softplus_lam, rate, state, seg_start, seg_pos0,
-                    seg_slot, chunks=None, seg_chunk0=None):
+                    seg_slot, chunks=None, seg_chunk0=None, gate_part=0):
     T, W = u.shape
     g = gates + gate_bias
+    if gate_part:          # block by block (r | i) -> (r | i) of all channels
+        g = g.reshape(T, W // gate_part, 2, gate_part).transpose(1, 2).reshape(T, 2 * W)
     a = torch.exp(-rate * torch.sigmoid(g[:, :W]) * softplus_lam)
     b = torch.sqrt(torch.clamp(1.0 - a * a, min=0.0)) * torch.sigmoid(g[:, W:]) * u.to(F32)
     z = y[:, :W].to(F32)
