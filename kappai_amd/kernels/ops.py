@@ -931,7 +931,10 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     _need(not (window and chunk) and (window or 0) >= 0 and chunk >= 0,
           "paged_attention: a sliding window or chunks, not both")
     if chunk:
-        window = -int(chunk)
+        # (while no position of the step has left the first chunk, a chunk is the whole past:
+        # the kernels' plain form, which pairs the tiles of a portion for equal work)
+        first_chunk_only = max_position is not None and 0 <= max_position < chunk
+        window = 0 if first_chunk_only else -int(chunk)
     if mods is not None and not mods.active():
         mods = None
     mods_c = mods.c_struct(H) if mods is not None else None
