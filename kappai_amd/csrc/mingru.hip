@@ -250,3 +250,122 @@ extern "C" int kappai_gated_unit_scan(const float* gates, const float* gate_bias
                                  n_chunks, carry, out, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------
+// A decode step of the real-gated unit in one kernel, for steps whose every segment is a single
+// row: the convolution over the request's history (and the history brought up to date), both
+// gates of a block, the recurrence and the gated output.  A block of threads takes a (row, block
+// of channels): u of the block's `part` channels is made and kept in LDS (rounded as the
+// convolution's own kernel stores it), a thread takes a row of the block's gate matrix (W [blocks,
+// 2 part, part]: the rows of r, then those of i), and a thread a channel finishes.
+//   proj [T, >= 2W] rows `stride` apart: (x | y) with biases added; taps [W, n], conv_bias [W],
+//   conv_state [slots, n - 1, W] oldest first; gate_bias [blocks, 2 part]; sp [W] = softplus(lam);
+//   state [slots, W]; seg_pos0 / seg_slot [T]; out [T, W] stored as proj is.
+// ---------------------------------------------------------------------------------------
+#define GU_STEP_THREADS 256
+__device__ __forceinline__ void gu_load8(const float* p, float (&w)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+}
+__device__ __forceinline__ void gu_load8(const bf16_t* p, float (&w)[8]) {
+  const uint4 u = *reinterpret_cast<const uint4*>(p);
+  const unsigned v[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    w[2 * k] = __uint_as_float(v[k] << 16);
+    w[2 * k + 1] = __uint_as_float(v[k] & 0xffff0000u);
+  }
+}
+
+template <typename TP>
+__global__ __launch_bounds__(GU_STEP_THREADS) void gated_unit_step_kernel(
+    const TP* __restrict__ proj, int stride, const float* __restrict__ taps, int n_taps,
+    const float* __restrict__ conv_bias, float* __restrict__ conv_state,
+    const TP* __restrict__ gate_w, const float* __restrict__ gate_bias,
+    const float* __restrict__ sp, float rate, float* __restrict__ state,
+    const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot, int W, int part,
+    TP* __restrict__ out) {
+  extern __shared__ float gu_lds[];
+  float* us = gu_lds;                 // [part]
+  float* gs = gu_lds + part;          // [2 part]
+  const int t = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int pos = seg_pos0[t], slot = seg_slot[t], keep = n_taps - 1;
+  const TP* row = proj + (size_t)t * stride;
+  float* hist = conv_state + (size_t)slot * keep * W;
+  for (int i = tid; i < part; i += GU_STEP_THREADS) {
+    const int c = b * part + i;
+    const float x = to_f32(row[c]);
+    const float* tp = taps + (size_t)c * n_taps;
+    float acc = tp[keep] * x;
+    float older[16];
+    for (int j = 0; j < keep; ++j) {
+      // entry j of the history is the token `keep - j` before this one
+      older[j] = keep - j <= pos ? hist[(size_t)j * W + c] : 0.f;
+      acc = fmaf(tp[j], older[j], acc);
+    }
+    for (int j = 0; j + 1 < keep; ++j) hist[(size_t)j * W + c] = older[j + 1];
+    if (keep > 0) hist[(size_t)(keep - 1) * W + c] = x;
+    TP stored;
+    from_f32(&stored, acc + conv_bias[c]);
+    us[i] = to_f32(stored);
+  }
+  __syncthreads();
+  // a thread a row of the block's gate matrix: its loads do not wait for one another, and the
+  // block's u is read from LDS by all lanes at once
+  const TP* wb = gate_w + (size_t)b * 2 * part * part;
+  for (int o = tid; o < 2 * part; o += GU_STEP_THREADS) {
+    const TP* wr = wb + (size_t)o * part;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    int i = 0;
+    if (part % 8 == 0 && ((uintptr_t)wb % 16) == 0) {
+      for (; i < part; i += 8) {
+        float w[8];
+        gu_load8(wr + i, w);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[k % 4] = fmaf(w[k], us[i + k], acc[k % 4]);
+      }
+    }
+    for (; i < part; ++i) acc[0] = fmaf(to_f32(wr[i]), us[i], acc[0]);
+    gs[o] = (acc[0] + acc[1]) + (acc[2] + acc[3]) + gate_bias[(size_t)b * 2 * part + o];
+  }
+  __syncthreads();
+  for (int i = tid; i < part; i += GU_STEP_THREADS) {
+    const int c = b * part + i;
+    const float la = -rate * sigmoid_f(gs[i]) * sp[c];
+    const float a = expf(la);
+    const float in = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f)) * sigmoid_f(gs[part + i]) * us[i];
+    float* st = state + (size_t)slot * W + c;
+    const float S = fmaf(a, pos > 0 ? *st : 0.f, in);
+    *st = S;
+    const float z = to_f32(row[W + c]);
+    const float g = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    from_f32(out + (size_t)t * W + c, S * g);
+  }
+}
+
+extern "C" int kappai_gated_unit_step(const void* proj, int stride, const float* taps, int n_taps,
+                                      const float* conv_bias, float* conv_state,
+                                      const void* gate_w, const float* gate_bias, const float* sp,
+                                      float rate, float* state, const int* seg_pos0,
+                                      const int* seg_slot, int T, int W, int blocks, int is_bf16,
+                                      void* out, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (W < 1 || blocks < 1 || blocks > 65535 || W % blocks || n_taps < 1 || n_taps > 17 ||
+      stride < 2 * W || W / blocks > 4096 || !conv_bias || !gate_bias || !sp ||
+      (n_taps > 1 && !conv_state))
+    return (int)hipErrorInvalidValue;
+  const int part = W / blocks;
+  const size_t lds = (size_t)3 * part * sizeof(float);
+  const dim3 grid(T, blocks);
+  if (is_bf16)
+    hipLaunchKernelGGL(gated_unit_step_kernel<bf16_t>, grid, dim3(GU_STEP_THREADS), lds, stream,
+                       (const bf16_t*)proj, stride, taps, n_taps, conv_bias, conv_state,
+                       (const bf16_t*)gate_w, gate_bias, sp, rate, state, seg_pos0, seg_slot, W,
+                       part, (bf16_t*)out);
+  else
+    hipLaunchKernelGGL(gated_unit_step_kernel<float>, grid, dim3(GU_STEP_THREADS), lds, stream,
+                       (const float*)proj, stride, taps, n_taps, conv_bias, conv_state,
+                       (const float*)gate_w, gate_bias, sp, rate, state, seg_pos0, seg_slot, W,
+                       part, (float*)out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

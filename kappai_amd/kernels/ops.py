@@ -1465,6 +1465,54 @@ def gated_unit_scan(gates: torch.Tensor, gate_bias: torch.Tensor, u: torch.Tenso
     return out
 
 
+GATED_UNIT_STEP_MAX_PART = 4096     # channels a block that the one-kernel decode step takes
+
+
+def gated_unit_step(proj: torch.Tensor, taps: torch.Tensor, conv_bias: torch.Tensor,
+                    conv_state: torch.Tensor, gate_w: torch.Tensor, gate_bias: torch.Tensor,
+                    softplus_lam: torch.Tensor, rate: float, state: torch.Tensor,
+                    seg_pos0: torch.Tensor, seg_slot: torch.Tensor) -> torch.Tensor:
+    """A step of single rows (row t is segment t) through the real-gated unit in one kernel:
+    ``conv_silu`` without activation, both gates of every block, ``gated_unit_scan`` and the
+    states brought up to date.  ``proj`` [T, >= 2W] = (x | y) with biases added (a view with a
+    row stride), ``taps`` [W, n] float32, ``conv_bias`` [W], ``conv_state`` [slots, n - 1, W],
+    ``gate_w`` [blocks, 2 part, part] stored as ``proj`` is (rows of r, then of i),
+    ``gate_bias`` [blocks * 2 part] float32, ``softplus_lam`` [W], ``state`` [slots, W].
+    Returns [T, W] as ``proj`` is stored."""
+    _gpu("proj", proj, (F32, BF16), contiguous=False)
+    _gpu("taps", taps, F32)
+    _gpu("conv_bias", conv_bias, F32)
+    _gpu("conv_state", conv_state, F32)
+    _gpu("gate_w", gate_w, proj.dtype)
+    _gpu("gate_bias", gate_bias, F32)
+    _gpu("softplus_lam", softplus_lam, F32)
+    _gpu("state", state, F32)
+    _gpu("seg_pos0", seg_pos0, I32)
+    _gpu("seg_slot", seg_slot, I32)
+    T = proj.shape[0]
+    W, n = taps.shape
+    _need(gate_w.dim() == 3 and gate_w.shape[1] == 2 * gate_w.shape[2]
+          and gate_w.shape[0] * gate_w.shape[2] == W,
+          lambda: f"gated_unit_step: gate matrices {tuple(gate_w.shape)} for {W} channels")
+    blocks, part = gate_w.shape[0], gate_w.shape[2]
+    _need(proj.dim() == 2 and proj.shape[1] >= 2 * W and proj.stride(1) == 1
+          and 1 <= n <= CONV_SILU_MAX_TAPS and part <= GATED_UNIT_STEP_MAX_PART
+          and conv_bias.shape == (W,) and tuple(conv_state.shape[1:]) == (n - 1, W)
+          and gate_bias.shape == (2 * W,) and softplus_lam.shape == (W,)
+          and state.dim() == 2 and state.shape[1] == W
+          and seg_pos0.shape[0] == T and seg_slot.shape[0] == T,
+          lambda: f"gated_unit_step: proj {tuple(proj.shape)}, taps {tuple(taps.shape)}, "
+                  f"conv_state {tuple(conv_state.shape)}, state {tuple(state.shape)}, "
+                  f"{seg_slot.shape[0]} segments")
+    out = torch.empty((T, W), dtype=proj.dtype, device=proj.device)
+    check(library("mingru").kappai_gated_unit_step(
+        _ptr(proj), _c_int(proj.stride(0)), _ptr(taps), _c_int(n), _ptr(conv_bias),
+        _ptr(conv_state), _ptr(gate_w), _ptr(gate_bias), _ptr(softplus_lam), _c_float(rate),
+        _ptr(state), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(W), _c_int(blocks),
+        _c_int(_is_bf16(proj.dtype)), _ptr(out), _stream()), "gated_unit_step")
+    return out
+
+
 # ---------------------------------------------------------------------------------------
 # differential attention: the two maps of a head as heads of the paged attention kernels
 # ---------------------------------------------------------------------------------------

@@ -98,6 +98,14 @@ class RealGatedUnit(Mixer):
             state = cache.state
             conv_state = torch.empty((state.shape[0], 0, C), dtype=torch.float32,
                                      device=state.device)
+        if (batch.max_segment_rows == 1
+                and C // self.blocks <= ops.GATED_UNIT_STEP_MAX_PART):
+            # single rows: convolution, gates, recurrence and gated output in one kernel
+            with profile.scope("scan"):
+                y = ops.gated_unit_step(proj, self.conv_taps, self.conv_bias, conv_state,
+                                        self.gate_w, self.gate_b, self.softplus_lam, self.rate,
+                                        state, batch.seg_pos0, batch.seg_slot)
+            return self.out.forward(y, partial_sums=True)
         with profile.scope("short_conv"):
             u = ops.conv_silu(proj, self.conv_taps, conv_state, batch.row_pos, batch.row_seg,
                               batch.seg_start, batch.seg_pos0, batch.seg_slot,

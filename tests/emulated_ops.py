@@ -635,6 +635,24 @@ def gated_unit_scan(gates, gate_bias, u, y, softplus_lam, rate, state, seg_start
     return out.to(u.dtype)
 
 
+GATED_UNIT_STEP_MAX_PART = 4096
+
+
+def gated_unit_step(proj, taps, conv_bias, conv_state, gate_w, gate_bias, softplus_lam, rate,
+                    state, seg_pos0, seg_slot):
+    T = proj.shape[0]
+    W = taps.shape[0]
+    part = gate_w.shape[2]
+    rows = torch.arange(T, dtype=torch.int32)
+    starts = torch.arange(T + 1, dtype=torch.int32)
+    u = conv_silu(proj, taps, conv_state, seg_pos0, rows, starts, seg_pos0, seg_slot,
+                  bias=conv_bias, activation=False)
+    gates = torch.empty((T, 2 * W), dtype=F32)
+    headwise_linear(u, part, gate_w, out=gates, out_head_stride=2 * part, out_dtype=F32)
+    return gated_unit_scan(gates, gate_bias, u, proj[:, W:], softplus_lam, rate, state, starts,
+                           seg_pos0, seg_slot, gate_part=part)
+
+
 def pair_norm_sum(a, b, scale_a=1.0, scale_b=1.0, weight_a=None, weight_b=None, eps=0.0):
     def side(x, w):
         x = x.to(F32)
@@ -698,7 +716,7 @@ ALL = ["add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale
        "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
        "output_norm_add", "projection_norm_store", "latent_store", "headwise_linear", "conv_silu",
        "matrix_state_recurrence", "head_norm_gate", "rotate_widen_store", "token_shift_mix", "tanh",
-       "gated_unit_scan", "pair_norm_sum", "stream_enter",
+       "gated_unit_scan", "gated_unit_step", "pair_norm_sum", "stream_enter",
        "embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
