@@ -619,9 +619,11 @@ def test_a_pair_of_mixers(dtype, tol, kind):
 # ---------------------------------------------------------------------------------------------
 # whole models
 # ---------------------------------------------------------------------------------------------
-LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [150, 52, 75]}
+LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [150, 52, 75],
+           "E": [300, 90]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58], "B": [66, 35, 90, 41, 23, 77, 50, 62, 88],
-                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [75, 52, 160, 41, 66, 38, 90]}
+                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [75, 52, 160, 41, 66, 38, 90],
+                 "E": [140, 52, 260, 41, 66, 90]}
 
 
 @pytest.fixture(scope="module")
@@ -661,7 +663,7 @@ def replay(model_dir, dtype, steps, index, max_tokens, out_dir, slots=4, graphs=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     """Every logit of every request.  The mixed family runs in a pool smaller than its requests

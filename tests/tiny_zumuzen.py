@@ -97,8 +97,21 @@ TINY_D = config(301, 100, 1e-5, [
 ], loop=(0, 4, 2))
 INIT_D = dict(seed=44, std=0.08, norm_jitter=0.05)
 
+# wider: the time mixing first, heads of 32 and 64 that the matrix cores take as they are, values
+# half as wide as keys, a real-gated unit of 256 channels in blocks of 64 (the matrix per block
+# on the matrix cores) and one of a single block of 128, the two middle layers passed twice
+TINY_E = config(500, 192, 1e-6, [
+    parallel_2(left(6, 3, 32, 32, 0.25, 40000.0, 16, 40, (3.0, 128, 16.0, 2.0)), 3, 64, 16, 1.2,
+               0.4, dense(256)),
+    rglru(256, 4, 4, dense(224)),
+    parallel(left(8, 2, 64, 32, 0.11, 200000.0, 64, 128), 4, 16, 48, [0.2, 0.7, 0.95, 0.999],
+             dense(160)),
+    rglru(128, 1, 3, None),
+], loop=(1, 3, 2))
+INIT_E = dict(seed=45, std=0.06, norm_jitter=0.05)
+
 TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C),
-        "D": (TINY_D, INIT_D)}
+        "D": (TINY_D, INIT_D), "E": (TINY_E, INIT_E)}
 
 
 def write_tiny(name: str, folder, **overrides):
