@@ -38,16 +38,29 @@ __global__ __launch_bounds__(LA_THREADS) void conv_silu_kernel(
   const int t = blockIdx.x;
   const int c = blockIdx.y * LA_THREADS + threadIdx.x;
   if (c >= C) return;
-  const int seg = row_seg[t], first = seg_start[seg], pos = row_pos[t];
-  const float* st = state + (size_t)seg_slot[seg] * (n_taps - 1) * C;
-  float acc = 0.f;
+  // The sum over the rows before this one as if all of them were the segment's own: these loads
+  // wait for no table, so they are on their way while the row's segment, its start and its slot
+  // are read one after the other.  Only the first rows of a segment take the other path.
+  float ahead = 0.f;
   for (int j = 0; j < n_taps; ++j) {
-    const int back = n_taps - 1 - j;          // how many tokens before this one
-    if (back > pos) continue;                 // before the start of the sequence: zero
-    float v;
-    if (t - back >= first) v = to_f32(x[(size_t)(t - back) * x_stride + c]);
-    else v = st[(size_t)(n_taps - 1 - (back - (t - first))) * C + c];
-    acc = fmaf(taps[(size_t)c * n_taps + j], v, acc);
+    const int tt = t - (n_taps - 1 - j);
+    if (tt >= 0) ahead = fmaf(taps[(size_t)c * n_taps + j], to_f32(x[(size_t)tt * x_stride + c]), ahead);
+  }
+  const int seg = row_seg[t], first = seg_start[seg];
+  float acc = 0.f;
+  if (t - (n_taps - 1) >= first) {
+    acc = ahead;
+  } else {
+    const int pos = row_pos[t];
+    const float* st = state + (size_t)seg_slot[seg] * (n_taps - 1) * C;
+    for (int j = 0; j < n_taps; ++j) {
+      const int back = n_taps - 1 - j;          // how many tokens before this one
+      if (back > pos) continue;                 // before the start of the sequence: zero
+      float v;
+      if (t - back >= first) v = to_f32(x[(size_t)(t - back) * x_stride + c]);
+      else v = st[(size_t)(n_taps - 1 - (back - (t - first))) * C + c];
+      acc = fmaf(taps[(size_t)c * n_taps + j], v, acc);
+    }
   }
   if (bias != nullptr) acc += bias[c];
   from_f32(out + (size_t)t * C + c, act ? acc * la_sigmoid(acc) : acc);
