@@ -12,6 +12,8 @@
 //                           parts are rotated and put behind the r places that the product with
 //                           the keys' up-projection fills (headwise_linear)
 //   headwise_linear         y[t, h, :] = W[h] x[t, h, :], a matrix per head
+//   head_norm_rotate_store  RMS norm of every q and k head by itself (one weight [d] for all
+//                           heads), rotation of the first places, heads of d and dv widened to D
 #include "common.h"
 
 #define AP_THREADS 256
@@ -379,6 +381,101 @@ extern "C" int kappai_rotate_widen_store(
     hipLaunchKernelGGL(rotate_widen_store_kernel<float>, dim3(T), dim3(AP_THREADS), 0, stream,
                        (const float*)proj, stride, cos_tab, sin_tab, rot_dims, rot_mode,
                        values_are_keys, (float*)k_pool, (float*)v_pool, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, d, dv, D, ps, (float*)q_out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// head_norm_rotate_store: grouped-query heads whose queries and keys (d) and values (dv) differ
+// in size.  Every q and k head is divided by the root mean square of its own d places and
+// multiplied by a weight [d] that all heads share (q_norm_w / k_norm_w; null: no norm); then the
+// first rot_dims places of the head turn by the row's position.  proj [T, H d + G d + G dv].
+// Queries leave as H heads of D (zeros behind d); keys and values go to the pools as G heads of
+// D.  A wave a head: the sum of squares stays in the wave.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(AP_THREADS) void head_norm_rotate_store_kernel(
+    const T* __restrict__ proj, int stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rot_dims, int rot_mode, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int dv, int D,
+    int ps, T* __restrict__ q_out) {
+  const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  constexpr int NW = AP_THREADS / WAVE;
+  const int pos = row_pos[t];
+  const T* row = proj + (size_t)t * stride;
+  const int nq = H * d, nk = G * d, half = rot_dims / 2;
+  const float* ct = cos_tab + (size_t)pos * half;
+  const float* st = sin_tab + (size_t)pos * half;
+  size_t page = 0;
+  const int slot = pos % ps;
+  if (k_pool != nullptr) page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
+  // heads 0 .. H - 1 are queries, H .. H + G - 1 keys, then the G value heads
+  for (int head = wave; head < H + 2 * G; head += NW) {
+    if (head >= H + G) {
+      if (k_pool == nullptr) continue;
+      const int g = head - H - G;
+      for (int e = lane; e < D; e += WAVE)
+        from_f32(v_pool + ((page * G + g) * D + e) * ps + slot,
+                 e < dv ? to_f32(row[nq + nk + g * dv + e]) : 0.f);
+      continue;
+    }
+    const bool is_q = head < H;
+    if (!is_q && k_pool == nullptr) continue;
+    const T* src = is_q ? row + head * d : row + nq + (head - H) * d;
+    const float* w = is_q ? q_norm_w : k_norm_w;
+    float r = 1.f;
+    if (w != nullptr) {
+      float ss = 0.f;
+      for (int e = lane; e < d; e += WAVE) { const float v = to_f32(src[e]); ss = fmaf(v, v, ss); }
+      r = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+    }
+    auto normed = [&](int e) -> float {
+      const float v = to_f32(src[e]);
+      return w != nullptr ? v * r * w[e] : v;
+    };
+    T* dst = is_q ? q_out + ((size_t)t * H + head) * D
+                  : k_pool + ((page * G + (head - H)) * ps + slot) * D;
+    for (int e = lane; e < D; e += WAVE) {
+      float v = 0.f;
+      if (e < d) {
+        v = normed(e);
+        if (e < rot_dims && rot_mode != 0) {
+          int j, partner;
+          bool first;
+          if (rot_mode == 1) { first = e < half; j = first ? e : e - half; partner = first ? e + half : e - half; }
+          else { first = (e & 1) == 0; j = e / 2; partner = e ^ 1; }
+          const float y = normed(partner), c = ct[j], s = st[j];
+          v = first ? v * c - y * s : v * c + y * s;
+        }
+      }
+      from_f32(dst + e, v);
+    }
+  }
+}
+
+extern "C" int kappai_head_norm_rotate_store(
+    const void* proj, int stride, const float* q_norm_w, const float* k_norm_w, float eps,
+    const float* cos_tab, const float* sin_tab, int rot_dims, int rot_mode, void* k_pool,
+    void* v_pool, const int* row_pos, const int* row_seg, const int* block_tables, int max_blocks,
+    int T, int H, int G, int d, int dv, int D, int ps, void* q_out, int is_bf16,
+    hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || d < 1 || dv < 1 || D < d || D < dv || ps < 1 || rot_dims < 0 ||
+      rot_dims > d || rot_dims % 2 || rot_mode < 0 || rot_mode > 2 ||
+      (rot_mode && rot_dims && (!cos_tab || !sin_tab)))
+    return (int)hipErrorInvalidValue;
+  if (rot_dims == 0) rot_mode = 0;
+  if (is_bf16)
+    hipLaunchKernelGGL(head_norm_rotate_store_kernel<bf16_t>, dim3(T), dim3(AP_THREADS), 0,
+                       stream, (const bf16_t*)proj, stride, q_norm_w, k_norm_w, eps, cos_tab,
+                       sin_tab, rot_dims, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos,
+                       row_seg, block_tables, max_blocks, H, G, d, dv, D, ps, (bf16_t*)q_out);
+  else
+    hipLaunchKernelGGL(head_norm_rotate_store_kernel<float>, dim3(T), dim3(AP_THREADS), 0, stream,
+                       (const float*)proj, stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,
+                       rot_dims, rot_mode, (float*)k_pool, (float*)v_pool, row_pos, row_seg,
                        block_tables, max_blocks, H, G, d, dv, D, ps, (float*)q_out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

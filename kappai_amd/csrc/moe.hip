@@ -26,8 +26,9 @@ extern "C" int kappai_moe_tile_rows() { return MOE_TILE_M; }
 // and are added in the order of the waves.  Then the first wave chooses.
 template <typename T, int VEC>
 __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
-    const T* __restrict__ x, int ldx, const float* __restrict__ router, int n_rows, int D, int E,
-    int top, int* __restrict__ idx, float* __restrict__ wts) {
+    const T* __restrict__ x, int ldx, const float* __restrict__ router,
+    const float* __restrict__ bias, int n_rows, int D, int E, int top, int* __restrict__ idx,
+    float* __restrict__ wts) {
   extern __shared__ float route_lds[];
   constexpr int NW = MOE_THREADS / WAVE;
   float* logits = route_lds;                       // [E]
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
     if (threadIdx.x < MOE_ROUTE_GROUP && e0 + threadIdx.x < E) {
       float sum = part[threadIdx.x * NW];
       for (int w = 1; w < NW; ++w) sum += part[threadIdx.x * NW + w];
-      logits[e0 + threadIdx.x] = sum;
+      logits[e0 + threadIdx.x] = bias ? sum + bias[e0 + threadIdx.x] : sum;
     }
     __syncthreads();
   }
@@ -108,15 +109,16 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
   }
 }
 
-extern "C" int kappai_moe_route(const void* x, int ldx, int x_is_bf16, const float* router, int T,
-                                int D, int E, int top, int* idx, float* wts, hipStream_t stream) {
+extern "C" int kappai_moe_route(const void* x, int ldx, int x_is_bf16, const float* router,
+                                const float* bias, int T, int D, int E, int top, int* idx,
+                                float* wts, hipStream_t stream) {
   if (T <= 0) return 0;
   if (top < 1 || top > MOE_MAX_TOP || top > E || E > 4096) return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)(E + MOE_ROUTE_GROUP * (MOE_THREADS / WAVE)) * sizeof(float);
   const bool vec = D % 4 == 0 && (uintptr_t)router % 16 == 0;
 #define MOE_ROUTE_LAUNCH(TT, V)                                                                 \
   hipLaunchKernelGGL((moe_route_kernel<TT, V>), dim3(T), dim3(MOE_THREADS), lds, stream,          \
-                     (const TT*)x, ldx, router, T, D, E, top, idx, wts)
+                     (const TT*)x, ldx, router, bias, T, D, E, top, idx, wts)
   if (x_is_bf16) {
     if (vec) MOE_ROUTE_LAUNCH(bf16_t, 4); else MOE_ROUTE_LAUNCH(bf16_t, 1);
   } else {
@@ -228,11 +230,13 @@ extern "C" int kappai_moe_plan(const int* idx, int P, int E, int n_tiles, int* s
 }
 
 __device__ __forceinline__ float silu_exact(float g) { return g / (1.0f + expf(-g)); }
+__device__ __forceinline__ float relu_squared(float z) { const float r = fmaxf(z, 0.f); return r * r; }
 
 // Half a tile (MOE_HALF_M slots) of one expert times MOE_TILE_N rows of its matrix, float sums on
 // the vector units (this is the 32-bit path, and the path of any shape).  GATED: the rows are
-// gathered from x by pair / top, two matrices, out = silu(g) * u in T; else the rows are the
-// slots of `a` themselves and out is float.
+// gathered from x by pair / top, two matrices, out = silu(g) * u in T; GATED == 2: gathered rows,
+// one matrix, out = relu(x W^T)^2 in T; else the rows are the slots of `a` themselves and out is
+// float.
 template <typename T, int GATED>
 __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
     const T* __restrict__ a, int lda, const T* __restrict__ w0, const T* __restrict__ w1, int N,
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
   if (e < 0) return;
   __shared__ float As[MOE_TILE_K][MOE_HALF_M + 1];
   __shared__ float W0s[MOE_TILE_K][MOE_TILE_N + 1];
-  __shared__ float W1s[GATED ? MOE_TILE_K : 1][MOE_TILE_N + 1];
+  __shared__ float W1s[GATED == 1 ? MOE_TILE_K : 1][MOE_TILE_N + 1];
   __shared__ int src_row[MOE_HALF_M];
   const int tid = threadIdx.x;
   if (tid < MOE_HALF_M) {
@@ -254,7 +258,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
   __syncthreads();
   const int n0 = blockIdx.y * MOE_TILE_N;
   const T* W0 = w0 + (size_t)e * N * K;
-  const T* W1 = GATED ? w1 + (size_t)e * N * K : nullptr;
+  const T* W1 = GATED == 1 ? w1 + (size_t)e * N * K : nullptr;
   const int ty = tid / 16, tx = tid % 16;
   float acc0[2][4] = {}, acc1[2][4] = {};
   const int am = tid / 8, ak = (tid % 8) * 4;       // this thread's piece of the A tile
@@ -271,7 +275,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
       const int k = k0 + wk + i, n = n0 + wn;
       const bool ok = n < N && k < K;
       W0s[wk + i][wn] = ok ? to_f32(W0[(size_t)n * K + k]) : 0.f;
-      if (GATED) W1s[wk + i][wn] = ok ? to_f32(W1[(size_t)n * K + k]) : 0.f;
+      if (GATED == 1) W1s[wk + i][wn] = ok ? to_f32(W1[(size_t)n * K + k]) : 0.f;
     }
     __syncthreads();
 #pragma unroll 8
@@ -282,7 +286,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
         const float b0 = W0s[k][tx + 16 * j];
         acc0[0][j] = fmaf(a0, b0, acc0[0][j]);
         acc0[1][j] = fmaf(a1, b0, acc0[1][j]);
-        if (GATED) {
+        if (GATED == 1) {
           const float b1 = W1s[k][tx + 16 * j];
           acc1[0][j] = fmaf(a0, b1, acc1[0][j]);
           acc1[1][j] = fmaf(a1, b1, acc1[1][j]);
@@ -300,8 +304,10 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
       if (n >= N) continue;
-      if (GATED)
+      if (GATED == 1)
         from_f32((T*)out_v + slot * N + n, silu_exact(acc0[i][j]) * acc1[i][j]);
+      else if (GATED == 2)
+        from_f32((T*)out_v + slot * N + n, relu_squared(acc0[i][j]));
       else
         ((float*)out_v)[slot * N + n] = acc0[i][j];
     }
@@ -318,10 +324,13 @@ extern "C" int kappai_moe_gemm(const void* a, int lda, const void* w0, const voi
 #define MOE_GEMM_LAUNCH(TT, G)                                                                  \
   hipLaunchKernelGGL((moe_gemm_kernel<TT, G>), grid, dim3(MOE_THREADS), 0, stream, (const TT*)a, \
                      lda, (const TT*)w0, (const TT*)w1, N, K, tile_expert, pair_of_slot, top, out)
+  if (gated < 0 || gated > 2) return (int)hipErrorInvalidValue;
   if (is_bf16) {
-    if (gated) MOE_GEMM_LAUNCH(bf16_t, 1); else MOE_GEMM_LAUNCH(bf16_t, 0);
+    if (gated == 1) MOE_GEMM_LAUNCH(bf16_t, 1); else if (gated == 2) MOE_GEMM_LAUNCH(bf16_t, 2);
+    else MOE_GEMM_LAUNCH(bf16_t, 0);
   } else {
-    if (gated) MOE_GEMM_LAUNCH(float, 1); else MOE_GEMM_LAUNCH(float, 0);
+    if (gated == 1) MOE_GEMM_LAUNCH(float, 1); else if (gated == 2) MOE_GEMM_LAUNCH(float, 2);
+    else MOE_GEMM_LAUNCH(float, 0);
   }
 #undef MOE_GEMM_LAUNCH
   KAPPAI_RETURN_LAUNCH_STATUS();
@@ -355,7 +364,7 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ w1, int N, int K, const int* __restrict__ tile_expert,
     const int* __restrict__ pair_of_slot, int top, int n_tiles, void* __restrict__ out_v) {
   constexpr int MT = MOE_TILE_M / 16;
-  constexpr int NG = GATED ? 2 : 1;
+  constexpr int NG = GATED == 1 ? 2 : 1;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int tile = BYROW ? blockIdx.x * MOE_MFMA_WAVES + wave : blockIdx.x;
   if (tile >= n_tiles) return;
@@ -384,7 +393,7 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
                                lane * 8
                          : ((size_t)e * N + (w_ok[j] ? n : 0)) * K + kg;
     wrow[0][j] = w0 + at;
-    if (GATED) wrow[1][j] = w1 + at;
+    if (GATED == 1) wrow[1][j] = w1 + at;
   }
   moe_f32x4_t acc[NG][NT][MT];
 #pragma unroll
@@ -446,9 +455,11 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
       for (int j = 0; j < NT; ++j) {
         const int n = n0 + 16 * j + col;
         if (n >= N) continue;
-        if (GATED)
+        if (GATED == 1)
           ((bf16_t*)out_v)[slot * N + n] =
-              f32_to_bf16(silu_exact(acc[0][j][t][v]) * acc[GATED ? 1 : 0][j][t][v]);
+              f32_to_bf16(silu_exact(acc[0][j][t][v]) * acc[GATED == 1 ? 1 : 0][j][t][v]);
+        else if (GATED == 2)
+          ((bf16_t*)out_v)[slot * N + n] = f32_to_bf16(relu_squared(acc[0][j][t][v]));
         else
           ((float*)out_v)[slot * N + n] = acc[0][j][t][v];
       }
@@ -475,8 +486,11 @@ extern "C" int kappai_moe_gemm_mfma(const void* a, int lda, const void* w0, cons
           : dim3(n_tiles, (N + 16 * NT_ * MOE_MFMA_WAVES - 1) / (16 * NT_ * MOE_MFMA_WAVES)),      \
       block, 0, stream, (const bf16_t*)a, lda, (const bf16_t*)w0, (const bf16_t*)w1, N, K,         \
       tile_expert, pair_of_slot, top, n_tiles, out)
-  if (gated) {
+  if (gated < 0 || gated > 2) return (int)hipErrorInvalidValue;
+  if (gated == 1) {
     if (few) { MOE_MFMA_LAUNCH(1, 1, 2, false); } else { MOE_MFMA_LAUNCH(1, 4, 1, true); }
+  } else if (gated == 2) {
+    if (few) { MOE_MFMA_LAUNCH(2, 2, 2, false); } else { MOE_MFMA_LAUNCH(2, 4, 1, true); }
   } else {
     if (few) { MOE_MFMA_LAUNCH(0, 2, 2, false); } else { MOE_MFMA_LAUNCH(0, 4, 1, true); }
   }
@@ -487,10 +501,19 @@ extern "C" int kappai_moe_gemm_mfma(const void* a, int lda, const void* w0, cons
 
 __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(
     const float* __restrict__ y, const int* __restrict__ slot_of_pair,
-    const float* __restrict__ wts, int top, int D, float* __restrict__ out) {
+    const float* __restrict__ wts, int top, int D, const void* __restrict__ also,
+    int also_is_bf16, int also_parts, size_t also_plane, float* __restrict__ out) {
   const int t = blockIdx.x;
   for (int n = threadIdx.x; n < D; n += MOE_THREADS) {
+    // what every row gets beside its experts (a shared expert's result: rows, or float planes
+    // of a product cut over its input dimension, added in order) comes first
     float acc = 0.f;
+    if (also != nullptr) {
+      const size_t at = (size_t)t * D + n;
+      if (also_is_bf16) acc = bf16_to_f32(((const bf16_t*)also)[at]);
+      else
+        for (int p = 0; p < also_parts; ++p) acc += ((const float*)also)[p * also_plane + at];
+    }
     for (int k = 0; k < top; ++k)
       acc = fmaf(wts[(size_t)t * top + k], y[(size_t)slot_of_pair[(size_t)t * top + k] * D + n],
                  acc);
@@ -499,9 +522,11 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(
 }
 
 extern "C" int kappai_moe_combine(const float* y, const int* slot_of_pair, const float* wts, int T,
-                                  int top, int D, float* out, hipStream_t stream) {
+                                  int top, int D, const void* also, int also_is_bf16,
+                                  int also_parts, float* out, hipStream_t stream) {
   if (T <= 0) return 0;
+  if (also && also_parts < 1) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(MOE_THREADS), 0, stream, y, slot_of_pair,
-                     wts, top, D, out);
+                     wts, top, D, also, also_is_bf16, also_parts, (size_t)T * D, out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -1,0 +1,216 @@
+// A residual stream kept in several copies ("hyper-connections"), the layer norm that reads it,
+// and small gates and caps around attention layers that use them.
+//
+//   hyper_step     one pass over a row's S copies x_1 .. x_S [T, S, W] (float32):
+//                    write:  x_t <- sum_s mix[s, t] x_s + out[t] * y     (all t from the old x_s)
+//                    read:   u = sum_s in[s] x_s;  rows = (u - mean) / sqrt(var + eps) * w
+//                  either half may be left out; `spread`: the copies do not exist yet and are all
+//                  the row of `source` [T, W] (the embedded rows); `rows`: only the listed rows
+//                  are read (and, with a write half, their new copies are not stored: the norm
+//                  before the output head).
+//   rows_rmsnorm   y = x / sqrt(mean(x^2) + eps) * w on the first n columns of strided rows
+//   sigmoid_gate   x[t, i] *= sigmoid(g[t, i / group])
+//   softcap_rows   x <- c tanh(x / c), in place, float32
+//   activate       out = relu(x)^2 (kind 0)
+#include "common.h"
+
+#define HS_THREADS 256
+#define HS_MAX_STREAMS 8
+
+// y of row t, column c: rows of TY, or P float planes [P, T, W] added in order
+template <typename TY>
+__device__ __forceinline__ float update_at(const TY* __restrict__ y, int parts, size_t plane,
+                                           size_t at) {
+  float v = to_f32(y[at]);
+  for (int p = 1; p < parts; ++p) v += to_f32(y[(size_t)p * plane + at]);
+  return v;
+}
+
+template <typename TY, typename TO>
+__global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
+    float* __restrict__ streams, const float* __restrict__ source, const TY* __restrict__ y,
+    int parts, const float* __restrict__ mix, const float* __restrict__ out_w,
+    const float* __restrict__ in_w, const float* __restrict__ norm_w, float eps,
+    const int* __restrict__ rows, int store, TO* __restrict__ normed, int T, int S, int W) {
+  extern __shared__ float hs_lds[];
+  float* u_row = hs_lds;                 // [W]
+  float* red = hs_lds + W;               // [16]
+  __shared__ float c_mix[HS_MAX_STREAMS * HS_MAX_STREAMS], c_out[HS_MAX_STREAMS],
+      c_in[HS_MAX_STREAMS];
+  const int t = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int tid = threadIdx.x;
+  if (tid < S * S && mix) c_mix[tid] = mix[tid];
+  if (tid < S && out_w) c_out[tid] = out_w[tid];
+  if (tid < S && in_w) c_in[tid] = in_w[tid];
+  __syncthreads();
+  const bool write = y != nullptr, read = normed != nullptr;
+  const size_t plane = (size_t)T * W;
+  float sum = 0.f;
+  for (int c = tid; c < W; c += HS_THREADS) {
+    float x[HS_MAX_STREAMS];
+#pragma unroll
+    for (int s = 0; s < HS_MAX_STREAMS; ++s)
+      if (s < S) x[s] = source ? source[(size_t)t * W + c] : streams[((size_t)t * S + s) * W + c];
+    if (write) {
+      const float yv = update_at(y, parts, plane, (size_t)t * W + c);
+      float nx[HS_MAX_STREAMS];
+#pragma unroll
+      for (int to = 0; to < HS_MAX_STREAMS; ++to)
+        if (to < S) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s = 0; s < HS_MAX_STREAMS; ++s)
+            if (s < S) acc = fmaf(c_mix[s * S + to], x[s], acc);
+          nx[to] = fmaf(c_out[to], yv, acc);
+        }
+#pragma unroll
+      for (int s = 0; s < HS_MAX_STREAMS; ++s)
+        if (s < S) {
+          x[s] = nx[s];
+          if (store) streams[((size_t)t * S + s) * W + c] = nx[s];
+        }
+    } else if (source && store) {
+#pragma unroll
+      for (int s = 0; s < HS_MAX_STREAMS; ++s)
+        if (s < S) streams[((size_t)t * S + s) * W + c] = x[s];
+    }
+    if (read) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < HS_MAX_STREAMS; ++s)
+        if (s < S) u = fmaf(c_in[s], x[s], u);
+      u_row[c] = u;
+      sum += u;
+    }
+  }
+  if (!read) return;
+  const float mean = block_sum(sum, red) / (float)W;
+  float sq = 0.f;
+  for (int c = tid; c < W; c += HS_THREADS) {
+    const float d = u_row[c] - mean;
+    sq = fmaf(d, d, sq);
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(sq, red) / (float)W + eps);
+  TO* dst = normed + (size_t)blockIdx.x * W;
+  for (int c = tid; c < W; c += HS_THREADS)
+    from_f32(dst + c, (u_row[c] - mean) * rstd * norm_w[c]);
+}
+
+extern "C" int kappai_hyper_step(float* streams, const float* source, const void* y,
+                                 int y_is_bf16, int parts, const float* mix, const float* out_w,
+                                 const float* in_w, const float* norm_w, float eps,
+                                 const int* rows, int n_rows, int store, void* normed,
+                                 int normed_is_bf16, int T, int S, int W, hipStream_t stream) {
+  const int blocks = rows ? n_rows : T;
+  if (blocks <= 0) return 0;
+  if (S < 1 || S > HS_MAX_STREAMS || W < 1 || parts < 1 || (!streams && !source) ||
+      (y && (!mix || !out_w)) || (normed && (!in_w || !norm_w)) || (store && !streams) ||
+      (rows && store))
+    return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)(W + 16) * sizeof(float);
+  if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
+#define HS_LAUNCH(TY, TO)                                                                        \
+  hipLaunchKernelGGL((hyper_step_kernel<TY, TO>), dim3(blocks), dim3(HS_THREADS), lds, stream,   \
+                     streams, source, (const TY*)y, parts, mix, out_w, in_w, norm_w, eps, rows,   \
+                     store, (TO*)normed, T, S, W)
+  if (y_is_bf16) {
+    if (normed_is_bf16) HS_LAUNCH(bf16_t, bf16_t); else HS_LAUNCH(bf16_t, float);
+  } else {
+    if (normed_is_bf16) HS_LAUNCH(float, bf16_t); else HS_LAUNCH(float, float);
+  }
+#undef HS_LAUNCH
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// A wave a row: the first n columns of a row of `x` (stride ldx), normed into `out` [T, n].
+template <typename T>
+__global__ __launch_bounds__(256) void rows_rmsnorm_kernel(
+    const T* __restrict__ x, int ldx, const float* __restrict__ w, float eps, int n_rows, int n,
+    T* __restrict__ out) {
+  const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (row >= n_rows) return;
+  const T* xr = x + (size_t)row * ldx;
+  float sq = 0.f;
+  for (int c = lane; c < n; c += WAVE) {
+    const float v = to_f32(xr[c]);
+    sq = fmaf(v, v, sq);
+  }
+  const float r = 1.0f / sqrtf(wave_sum(sq) / (float)n + eps);
+  for (int c = lane; c < n; c += WAVE)
+    from_f32(out + (size_t)row * n + c, to_f32(xr[c]) * r * w[c]);
+}
+
+extern "C" int kappai_rows_rmsnorm(const void* x, int ldx, const float* w, float eps, int T,
+                                   int n, void* out, int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (n < 1 || ldx < n) return (int)hipErrorInvalidValue;
+  const dim3 grid((T + 3) / 4), block(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(rows_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, ldx,
+                       w, eps, T, n, (bf16_t*)out);
+  else
+    hipLaunchKernelGGL(rows_rmsnorm_kernel<float>, grid, block, 0, stream, (const float*)x, ldx, w,
+                       eps, T, n, (float*)out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ x, const T* __restrict__ g, int ldg, int n,
+                                    int group, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / n;
+  const int c = (int)(i - t * n);
+  const float z = to_f32(g[t * ldg + c / group]);
+  from_f32(x + i, to_f32(x[i]) / (1.0f + expf(-z)));
+}
+
+extern "C" int kappai_sigmoid_gate(void* x, const void* g, int ldg, int T, int n, int group,
+                                   int is_bf16, hipStream_t stream) {
+  const size_t total = (size_t)T * n;
+  if (total == 0) return 0;
+  if (group < 1 || n % group) return (int)hipErrorInvalidValue;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (is_bf16)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                       (bf16_t*)x, (const bf16_t*)g, ldg, n, group, total);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)x,
+                       (const float*)g, ldg, n, group, total);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+__global__ void softcap_rows_kernel(float* __restrict__ x, float cap, float inv, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] * inv);
+}
+
+extern "C" int kappai_softcap_rows(float* x, long n, float cap, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(softcap_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                     x, cap, 1.0f / cap, (size_t)n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+__global__ void activate_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float r = fmaxf(to_f32(in[i]), 0.f);
+  from_f32(out + i, r * r);
+}
+
+extern "C" int kappai_activate(const void* in, void* out, long n, int kind, int is_bf16,
+                               hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (kind != 0) return (int)hipErrorInvalidValue;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (is_bf16)
+    hipLaunchKernelGGL(activate_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                       (const bf16_t*)in, (bf16_t*)out, (size_t)n);
+  else
+    hipLaunchKernelGGL(activate_kernel<float>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)in, (float*)out, (size_t)n);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

@@ -27,7 +27,7 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-f
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
 LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine", "engine_api",
-             "groupnorm", "mingru", "diffattn", "moe", "attn_prep", "linear_attention"]
+             "groupnorm", "mingru", "diffattn", "moe", "attn_prep", "linear_attention", "streams"]
 # libraries made of more sources than the one of their own name
 EXTRA_SOURCES = {"engine": ["engine_parts"]}
 

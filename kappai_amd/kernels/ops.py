@@ -1574,12 +1574,16 @@ def diff_combine(ctx: torch.Tensor, n_heads: int, n_kv_heads: int, vdim: int, he
 MOE_MAX_TOP = 16
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, top: int):
-    """Router logits ``x router^T`` in float32, the ``top`` largest of a row chosen (the lowest
-    index wins a tie), weights = softmax over the chosen logits.  Returns (experts [T, top] int32,
-    weights [T, top] float32), the largest first."""
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int,
+              bias: Optional[torch.Tensor] = None):
+    """Router logits ``x router^T (+ bias)`` in float32, the ``top`` largest of a row chosen (the
+    lowest index wins a tie), weights = softmax over the chosen logits.  Returns (experts [T, top]
+    int32, weights [T, top] float32), the largest first."""
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("router", router, F32)
+    if bias is not None:
+        _gpu("bias", bias, F32)
+        _need(bias.shape == (router.shape[0],), lambda: f"moe_route: bias {tuple(bias.shape)}")
     T, D = x.shape
     E = router.shape[0]
     _need(router.shape == (E, D) and x.stride(1) == 1 and 1 <= top <= min(E, MOE_MAX_TOP),
@@ -1587,8 +1591,9 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, top: int):
     idx = torch.empty((T, top), dtype=I32, device=x.device)
     wts = torch.empty((T, top), dtype=F32, device=x.device)
     check(library("moe").kappai_moe_route(
-        _ptr(x), _c_int(x.stride(0)), _c_int(_is_bf16(x.dtype)), _ptr(router), _c_int(T),
-        _c_int(D), _c_int(E), _c_int(top), _ptr(idx), _ptr(wts), _stream()), "moe_route")
+        _ptr(x), _c_int(x.stride(0)), _c_int(_is_bf16(x.dtype)), _ptr(router), _ptr(bias),
+        _c_int(T), _c_int(D), _c_int(E), _c_int(top), _ptr(idx), _ptr(wts), _stream()),
+        "moe_route")
     return idx, wts
 
 
@@ -1697,6 +1702,34 @@ def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
     return out
 
 
+def moe_experts_activated(x: torch.Tensor, w_up: torch.Tensor, plan: MoePlan) -> torch.Tensor:
+    """``relu(x Wu[e]^T)^2`` for every slot of the plan ([slots, F], the dtype of ``x``; empty
+    slots are left unwritten): experts of one matrix in, no gate.  ``w_up``: [E, F, D]."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    E, F, D = w_up.shape
+    w_up, frag = _moe_matrix(w_up)
+    _gpu("w_up", w_up, x.dtype)
+    _need(x.shape[1] == D and x.stride(1) == 1,
+          lambda: f"moe_experts_activated: x {tuple(x.shape)}, matrices {(E, F, D)}")
+    out = torch.empty((plan.n_tiles * plan.tile_rows, F), dtype=x.dtype, device=x.device)
+    mfma = _moe_on_matrix_cores(x, x.stride(0), D, w_up)
+    _need(mfma or not frag, "moe_experts_activated: matrices in fragment order need bfloat16 "
+          "rows with 16-byte aligned starts")
+    if mfma:
+        check(library("moe").kappai_moe_gemm_mfma(
+            _ptr(x), _c_int(x.stride(0)), _ptr(w_up), _vp(0), _c_int(F), _c_int(D),
+            _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top),
+            _c_int(plan.n_tiles), _ptr(out), _c_int(2), _c_int(_moe_few(plan)), _c_int(frag),
+            _stream()), "moe_gemm_mfma (up, squared relu)")
+        return out
+    check(library("moe").kappai_moe_gemm(
+        _ptr(x), _c_int(x.stride(0)), _ptr(w_up), _vp(0), _c_int(F), _c_int(D),
+        _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top), _c_int(plan.n_tiles),
+        _ptr(out), _c_int(2), _c_int(_is_bf16(x.dtype)), _stream()),
+        "moe_gemm (up, squared relu)")
+    return out
+
+
 def moe_experts_down(act: torch.Tensor, w_down: torch.Tensor, plan: MoePlan) -> torch.Tensor:
     """``act W_down[e]^T`` for every slot of the plan: float32 [slots, D]."""
     _gpu("act", act, (F32, BF16))
@@ -1722,16 +1755,27 @@ def moe_experts_down(act: torch.Tensor, w_down: torch.Tensor, plan: MoePlan) -> 
     return out
 
 
-def moe_combine(y: torch.Tensor, weights: torch.Tensor, plan: MoePlan) -> torch.Tensor:
-    """``out[t] = sum_k weights[t, k] * y[slot of (t, k)]`` in the order of k: float32 [T, D]."""
+def moe_combine(y: torch.Tensor, weights: torch.Tensor, plan: MoePlan,
+                also: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t] = (also[t] +) sum_k weights[t, k] * y[slot of (t, k)]`` in the order of k: float32
+    [T, D].  ``also``: what every row gets beside its experts, [T, D] in float32 or bfloat16, or
+    float32 partial sums [S, T, D] (added in order)."""
     _gpu("y", y, F32)
     _gpu("weights", weights, F32)
     T, top = weights.shape
     D = y.shape[1]
     _need(top == plan.top and plan.slot_of_pair.shape[0] == T * top, "moe_combine: another plan")
+    parts = 1
+    if also is not None:
+        _gpu("also", also, (F32, BF16))
+        if also.dim() == 3:
+            _need(also.dtype == F32, "moe_combine: partial sums are float32")
+            parts = also.shape[0]
+        _need(tuple(also.shape[-2:]) == (T, D), lambda: f"moe_combine: also {tuple(also.shape)}")
     out = torch.empty((T, D), dtype=F32, device=y.device)
     check(library("moe").kappai_moe_combine(
         _ptr(y), _ptr(plan.slot_of_pair), _ptr(weights), _c_int(T), _c_int(top), _c_int(D),
+        _ptr(also), _c_int(_is_bf16(also.dtype) if also is not None else 0), _c_int(parts),
         _ptr(out), _stream()), "moe_combine")
     return out
 
@@ -1903,6 +1947,57 @@ def rotate_widen_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim: i
         _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
         _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size),
         _ptr(q), _c_int(_is_bf16(proj.dtype)), _stream()), "rotate_widen_store")
+    return q
+
+
+def head_norm_rotate_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int,
+                           vdim: int, head_size: int, q_norm_w: Optional[torch.Tensor],
+                           k_norm_w: Optional[torch.Tensor], eps: float,
+                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                           rot_dims: int, rot_mode: int, k_pool: torch.Tensor,
+                           v_pool: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor,
+                           block_tables: torch.Tensor, page_size: int) -> torch.Tensor:
+    """From ``proj`` [T, H dim + G dim + G vdim (+ more)]: every q and k head divided by the root
+    mean square of its own ``dim`` places and multiplied by a weight [dim] that the heads share
+    (None: no norm), then the first ``rot_dims`` places turned by the row's position (tables and
+    ``rot_mode`` as ``rotate_widen_store``).  Returns queries [T, H head_size] (zeros behind
+    ``dim``); keys and values go to pools made for G kv heads of ``head_size``."""
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    _gpu("proj", proj, (F32, BF16), contiguous=False)
+    T = proj.shape[0]
+    need = H * d + G * d + G * dv
+    _need(proj.dim() == 2 and proj.shape[1] >= need and proj.stride(1) == 1,
+          lambda: f"head_norm_rotate_store: proj {tuple(proj.shape)} holds fewer than {need} "
+                  "columns")
+    _need(H % G == 0 and d <= D and dv <= D,
+          lambda: f"head_norm_rotate_store: {H} heads over {G}, sizes {d} and {dv} in heads of {D}")
+    for name, w in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if w is not None:
+            _gpu(name, w, F32)
+            _need(w.shape == (d,), lambda: f"{name}: {tuple(w.shape)}, expected ({d},)")
+    if rot_mode != ROT_NONE and rot_dims:
+        _gpu("cos", cos, F32)
+        _gpu("sin", sin, F32)
+        _need(rot_dims % 2 == 0 and rot_dims <= d and cos.shape == sin.shape and cos.dim() == 2
+              and cos.shape[1] == rot_dims // 2,
+              lambda: f"head_norm_rotate_store: tables {tuple(cos.shape)} for {rot_dims} places "
+                      f"of {d}")
+    else:
+        rot_dims, rot_mode, cos, sin = 0, ROT_NONE, None, None
+    _gpu("k_pool", k_pool, proj.dtype)
+    _gpu("v_pool", v_pool, proj.dtype)
+    _check_pools(k_pool, v_pool, G, page_size, D)
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("block_tables", block_tables)):
+        _gpu(name, t, I32)
+    _need(row_pos.shape[0] == T and row_seg.shape[0] == T and block_tables.dim() == 2,
+          "head_norm_rotate_store: row tables do not fit the batch")
+    q = torch.empty((T, H * D), dtype=proj.dtype, device=proj.device)
+    check(library("attn_prep").kappai_head_norm_rotate_store(
+        _ptr(proj), _c_int(proj.stride(0)), _ptr(q_norm_w), _ptr(k_norm_w), _c_float(eps),
+        _ptr(cos), _ptr(sin), _c_int(rot_dims), _c_int(rot_mode), _ptr(k_pool), _ptr(v_pool),
+        _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
+        _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size),
+        _ptr(q), _c_int(_is_bf16(proj.dtype)), _stream()), "head_norm_rotate_store")
     return q
 
 
@@ -2205,4 +2300,128 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
         _c_int(gate_kind), _c_int(T), _c_int(H), _c_int(dv),
         _c_int(dv if weight.dim() == 2 else 0), _ptr(out),
         _c_int(_is_bf16(out_dtype)), _stream()), "head_norm_gate")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# a residual stream kept in several copies, its layer norm, gates and caps
+# ---------------------------------------------------------------------------------------
+HYPER_MAX_STREAMS = 8
+
+
+def hyper_step(streams: Optional[torch.Tensor], n_streams: int, width: int, source=None, y=None,
+               mix=None, out_w=None, in_w=None, norm_w=None, eps: float = 0.0, rows=None,
+               rows_dtype=None, store: bool = True) -> Optional[torch.Tensor]:
+    """One pass over the copies of the stream, ``streams`` [T, S, W] float32, in place.
+
+    Write half (``y``, ``mix`` [S, S] indexed [from, to], ``out_w`` [S]): every copy becomes
+    ``x_t <- sum_s mix[s, t] x_s + out_w[t] * y``, all from the old copies; ``y`` is [T, W] in
+    float32 or bfloat16, or float32 partial sums [P, T, W] added in order.  Read half (``in_w``
+    [S], ``norm_w`` [W], ``rows_dtype``): ``u = sum_s in_w[s] x_s`` of the new copies passes a
+    layer norm without bias, ``(u - mean) / sqrt(var + eps) * norm_w``, and is returned as
+    [T, W] in ``rows_dtype``.  ``source`` [T, W]: the copies do not exist yet and are all this
+    row (they are then written to ``streams`` when ``store``).  ``rows`` (int32): the read half
+    runs for these rows only, and the new copies are not stored."""
+    S, W = n_streams, width
+    _need(1 <= S <= HYPER_MAX_STREAMS, lambda: f"hyper_step: {S} copies of the stream; the kernel "
+                                               f"takes 1 to {HYPER_MAX_STREAMS}")
+    if streams is not None:
+        _gpu("streams", streams, F32)
+        _need(streams.dim() == 3 and tuple(streams.shape[1:]) == (S, W),
+              lambda: f"hyper_step: streams {tuple(streams.shape)} for {S} copies of {W}")
+    if source is not None:
+        _gpu("source", source, F32)
+        _need(source.dim() == 2 and source.shape[1] == W,
+              lambda: f"hyper_step: source {tuple(source.shape)}")
+    _need(streams is not None or source is not None, "hyper_step: nothing to read")
+    T = streams.shape[0] if streams is not None else source.shape[0]
+    _need(source is None or streams is None or source.shape[0] == T, "hyper_step: source rows")
+    parts = 1
+    if y is not None:
+        _gpu("y", y, (F32, BF16))
+        if y.dim() == 3:
+            _need(y.dtype == F32, "hyper_step: partial sums are float32")
+            parts = y.shape[0]
+        _need(tuple(y.shape[-2:]) == (T, W), lambda: f"hyper_step: y {tuple(y.shape)}")
+        _gpu("mix", mix, F32)
+        _gpu("out_w", out_w, F32)
+        _need(tuple(mix.shape) == (S, S) and tuple(out_w.shape) == (S,),
+              lambda: f"hyper_step: mix {tuple(mix.shape)}, out {tuple(out_w.shape)}")
+    normed = None
+    n_rows = T
+    if rows is not None:
+        _gpu("rows", rows, I32)
+        n_rows = rows.shape[0]
+        store = False
+    if rows_dtype is not None:
+        _gpu("in_w", in_w, F32)
+        _gpu("norm_w", norm_w, F32)
+        _need(tuple(in_w.shape) == (S,) and tuple(norm_w.shape) == (W,),
+              lambda: f"hyper_step: in {tuple(in_w.shape)}, norm weight {tuple(norm_w.shape)}")
+        normed = torch.empty((n_rows, W), dtype=rows_dtype, device=(
+            streams if streams is not None else source).device)
+    store = bool(store and streams is not None and (y is not None or source is not None))
+    check(library("streams").kappai_hyper_step(
+        _ptr(streams), _ptr(source), _ptr(y), _c_int(_is_bf16(y.dtype) if y is not None else 0),
+        _c_int(parts), _ptr(mix if y is not None else None),
+        _ptr(out_w if y is not None else None), _ptr(in_w if normed is not None else None),
+        _ptr(norm_w if normed is not None else None), _c_float(eps), _ptr(rows), _c_int(n_rows),
+        _c_int(1 if store else 0), _ptr(normed),
+        _c_int(_is_bf16(rows_dtype) if normed is not None else 0), _c_int(T), _c_int(S),
+        _c_int(W), _stream()), "hyper_step")
+    return normed
+
+
+def rows_rmsnorm(x: torch.Tensor, n: int, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """The first ``n`` columns of every row of ``x`` (rows may be strided) divided by their root
+    mean square (eps inside the root) and multiplied by ``weight`` [n]: a new [T, n] as ``x`` is
+    stored; sums in float32."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("weight", weight, F32)
+    _need(x.dim() == 2 and x.stride(1) == 1 and 1 <= n <= x.shape[1] and weight.shape == (n,),
+          lambda: f"rows_rmsnorm: x {tuple(x.shape)}, {n} columns, weight {tuple(weight.shape)}")
+    out = torch.empty((x.shape[0], n), dtype=x.dtype, device=x.device)
+    check(library("streams").kappai_rows_rmsnorm(
+        _ptr(x), _c_int(x.stride(0)), _ptr(weight), _c_float(eps), _c_int(x.shape[0]), _c_int(n),
+        _ptr(out), _c_int(_is_bf16(x.dtype)), _stream()), "rows_rmsnorm")
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, gate: torch.Tensor, group: int) -> torch.Tensor:
+    """``x[t, i] *= sigmoid(gate[t, i // group])`` in place; ``x`` [T, n] contiguous, ``gate``
+    [T, n / group] in the same dtype (rows may be strided).  ``group`` 1: a gate a channel; the
+    head size: a gate a head."""
+    _gpu("x", x, (F32, BF16))
+    _gpu("gate", gate, x.dtype, contiguous=False)
+    T, n = x.shape
+    _need(group >= 1 and n % group == 0 and gate.dim() == 2 and gate.shape[0] == T
+          and gate.shape[1] >= n // group and gate.stride(1) == 1,
+          lambda: f"sigmoid_gate: x {tuple(x.shape)}, gate {tuple(gate.shape)}, groups of {group}")
+    check(library("streams").kappai_sigmoid_gate(
+        _ptr(x), _ptr(gate), _c_int(gate.stride(0)), _c_int(T), _c_int(n), _c_int(group),
+        _c_int(_is_bf16(x.dtype)), _stream()), "sigmoid_gate")
+    return x
+
+
+def softcap_rows(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place; float32."""
+    _gpu("x", x, F32)
+    _need(cap > 0.0, lambda: f"softcap_rows: a cap of {cap}")
+    check(library("streams").kappai_softcap_rows(_ptr(x), _c_long(x.numel()), _c_float(cap),
+                                                 _stream()), "softcap_rows")
+    return x
+
+
+ACT_RELU_SQUARED = 0
+
+
+def activate(x: torch.Tensor, kind: int = ACT_RELU_SQUARED) -> torch.Tensor:
+    """An activation without a gate on every element, stored as ``x`` is: ``ACT_RELU_SQUARED``,
+    ``relu(x)^2``."""
+    _gpu("x", x, (F32, BF16))
+    _need(kind == ACT_RELU_SQUARED, lambda: f"activate: unknown activation {kind}")
+    out = torch.empty_like(x)
+    check(library("streams").kappai_activate(
+        _ptr(x), _ptr(out), _c_long(x.numel()), _c_int(kind), _c_int(_is_bf16(x.dtype)),
+        _stream()), "activate")
     return out

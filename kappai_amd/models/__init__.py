@@ -10,6 +10,7 @@ from ..weights.loader import check_and_load, parse_dtype, tensor_shapes
 from . import dapipel  # noqa: F401  (registers Dapipel)
 from . import dukolorn  # noqa: F401  (registers Dukolorn)
 from . import lfm2  # noqa: F401  (registers Lfm2ForCausalLM)
+from . import sibodra  # noqa: F401  (registers Sibodra)
 from . import zumuzen  # noqa: F401  (registers Zumuzen)
 from .base import LayerCall, Model
 

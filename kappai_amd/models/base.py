@@ -152,6 +152,8 @@ class Model:
         calls = []
         if self.embedding_norm is not None:
             return None            # the walk from C knows no norm between embedding and layers
+        if getattr(self.head, "softcap", 0.0):
+            return None            # nor a cap on the logits
         if any(call.enters is not None for call in self.schedule):
             return None            # nor parts that work on the stream between two blocks
         for ci, call in enumerate(self.schedule):

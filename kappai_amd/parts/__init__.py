@@ -1,7 +1,7 @@
 from .attention import GroupedQueryAttention
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, FeedForward,
                    Hidden, Mixer, Norm, Part, PositionEncoding, make_part, register_part)
-from .block import ConvInputBlock, OutputNormBlock, PreNormBlock
+from .block import ConvInputBlock, HyperConnectionBlock, OutputNormBlock, PreNormBlock
 from .diff_attention import DifferentialAttention
 from .embedding import OutputHead, TokenEmbedding
 from .feed_forward import SwiGLU
@@ -14,7 +14,7 @@ from .linear_attention import (BonusTimeMixing, FixedDecayAttention, GatedDeltaR
                                GatedLinearAttention)
 from .mingru import MinGRU
 from .moe import MixtureOfExperts
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 from .parallel import ParallelMixer
 from .passes import PassEntry
 from .positions import LearnedPositions
@@ -30,4 +30,4 @@ __all__ = ["GroupedQueryAttention", "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS"
            "ShortInputConv", "MinGRU", "MixtureOfExperts", "LearnedPositions", "OutputNormBlock",
            "LatentAttention", "GatedDeltaRule", "GatedLinearAttention", "ParallelMixer",
            "ScoredAttention", "RealGatedUnit", "BonusTimeMixing", "FixedDecayAttention",
-           "PassEntry"]
+           "PassEntry", "HyperConnectionBlock", "LayerNorm"]

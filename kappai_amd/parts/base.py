@@ -177,6 +177,17 @@ class WeightedTerms:
     scale_b: float
 
 
+@dataclass
+class StreamUpdate:
+    """A sublayer's result that a stream kept in several copies has not taken yet: every copy
+    becomes ``x_t <- sum_s mix[s, t] x_s + out[t] * y``.  ``y``: [T, width] or float32 partial
+    sums [S, T, width]; ``mix`` [copies, copies] indexed [from, to] and ``out`` [copies] float32.
+    The pass that reads the stream next (``parts.norm.LayerNorm.read_streams``) applies it."""
+    y: torch.Tensor
+    mix: torch.Tensor
+    out: torch.Tensor
+
+
 class Block(Part):
     """An arrangement of parts around the residual stream."""
 

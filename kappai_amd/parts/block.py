@@ -9,7 +9,9 @@ from ..kernels import ops
 from ..weights.spec import TensorSpec
 from ctypes import Structure
 
-from .base import Block, FeedForward, Hidden, Mixer, Norm, register_part, summed_delta
+from .base import (Block, FeedForward, Hidden, Mixer, Norm, StreamUpdate, register_part,
+                   summed_delta)
+from ..weights.spec import INIT_CONNECT, VECTOR
 from .cdesc import NormPartDesc, PartDesc, defined_together
 
 
@@ -281,3 +283,120 @@ class OutputNormBlock(Block):
 
 
 register_part("block", "output_norm", OutputNormBlock)
+
+
+class HyperConnectionBlock(Block):
+    """A pre-norm layer around a residual stream kept in ``streams`` copies x_1 .. x_S
+    ("hyper-connections"; all copies start as the embedded row).  Sublayer q (1: the mixer, 2: the
+    feed-forward) reads ``u = sum_s in_q[s] x_s`` through its norm, and its result y goes back as
+
+        x_t <- sum_s mix_q[s, t] x_s + out_q[t] * y        (all t at once, from the old copies)
+
+    with ``in_q`` [S], ``out_q`` [S] and ``mix_q`` [S, S] (indexed [from, to]) from the file
+    (``<prefix>hc<q>.in|out|mix``).  ``learned`` False: one copy with in = out = mix = 1, the
+    plain residual sum, and no such tensors.  After the last layer the stream is the copies' sum,
+    which is what the model's last norm (``parts.norm.LayerNorm.add_norm``) reads.
+
+    A sublayer's result is not applied when it is made: it travels as a ``StreamUpdate`` to the
+    pass that reads the stream next, so each sublayer costs ONE pass over the copies (apply the
+    update before, sum for this sublayer, normalise).  The norms must know ``read_streams``."""
+
+    def __init__(self, prefix: str, streams: int, width: int, mixer_norm: Norm, mixer: Mixer,
+                 ffn_norm: Norm = None, feed_forward: FeedForward = None, learned: bool = True,
+                 names=None):
+        n = {"mixer": "hc1.", "feed_forward": "hc2.", "in": "in", "out": "out", "mix": "mix"}
+        n.update(names or {})
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        if not 1 <= streams <= ops.HYPER_MAX_STREAMS:
+            raise ValueError(f"{prefix}: {streams} copies of the stream; the kernel takes 1 to "
+                             f"{ops.HYPER_MAX_STREAMS}")
+        if not learned and streams != 1:
+            raise ValueError(f"{prefix}: {streams} copies of the stream need connection weights")
+        for norm in (mixer_norm, ffn_norm):
+            if norm is not None and not hasattr(norm, "read_streams"):
+                raise ValueError(f"{type(norm).__name__} cannot read a stream kept in copies (no "
+                                 "read_streams)")
+        self.S, self.width, self.learned = int(streams), int(width), bool(learned)
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.ffn_norm, self.feed_forward = ffn_norm, feed_forward
+        self._names = {q: {k: prefix + n[q] + n[k] for k in ("in", "out", "mix")}
+                       for q in ("mixer", "feed_forward")}
+        self.weights = {}        # sublayer -> (in [S], out [S], mix [S, S]) float32
+
+    def _parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+                     if p is not None)
+
+    def _sublayers(self):
+        return ("mixer",) if self.feed_forward is None else ("mixer", "feed_forward")
+
+    @property
+    def capturable(self) -> bool:
+        return all(p.capturable for p in self._parts())
+
+    @property
+    def step_tables(self):
+        out = []
+        for p in self._parts():
+            asked = p.step_tables
+            if asked is not None:
+                out += list(asked) if isinstance(asked, (list, tuple)) else [asked]
+        return out
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [s for p in self._parts() for s in p.tensor_specs()]
+        if self.learned:
+            for q in self._sublayers():
+                nm = self._names[q]
+                specs += [TensorSpec(nm["in"], (self.S,), VECTOR, INIT_CONNECT),
+                          TensorSpec(nm["out"], (self.S,), VECTOR, INIT_CONNECT),
+                          TensorSpec(nm["mix"], (self.S, self.S), VECTOR, INIT_CONNECT)]
+        return specs
+
+    def unused_tensor_names(self) -> List[str]:
+        """What a file may hold for the feed-forward this layer does not have."""
+        if self.feed_forward is not None or not self.learned:
+            return []
+        return list(self._names["feed_forward"].values())
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self._parts():
+            p.bind(tensors)
+        for q in self._sublayers():
+            if self.learned:
+                nm = self._names[q]
+                self.weights[q] = tuple(tensors[nm[k]].to(torch.float32).contiguous()
+                                        for k in ("in", "out", "mix"))
+            else:
+                one = self.mixer_norm.ones
+                self.weights[q] = (one(1), one(1), one(1, 1))
+
+    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
+        streams, pending = h.resid, h.delta
+        w_in, w_out, w_mix = self.weights["mixer"]
+        if streams.dim() == 2:
+            # what the embedding left: every copy starts as that row
+            if pending is not None:
+                raise ValueError("an update is pending on a stream that has no copies yet")
+            source = streams
+            streams = torch.empty((source.shape[0], self.S, self.width), dtype=torch.float32,
+                                  device=source.device)
+            x = self.mixer_norm.read_streams(streams, w_in, source=source)
+        else:
+            if pending is not None and not isinstance(pending, StreamUpdate):
+                raise ValueError("a stream kept in copies takes its updates as StreamUpdate")
+            x = self.mixer_norm.read_streams(streams, w_in, pending=pending)
+        mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
+        update = StreamUpdate(mixed, w_mix, w_out)
+        if self.feed_forward is None:
+            return Hidden(streams, update)
+        w_in, w_out, w_mix = self.weights["feed_forward"]
+        x = self.ffn_norm.read_streams(streams, w_in, pending=update)
+        return Hidden(streams, StreamUpdate(self.feed_forward.forward(x, batch), w_mix, w_out))
+
+    def weight_bytes(self) -> int:
+        return sum(p.weight_bytes() for p in self._parts())
+
+
+register_part("block", "hyper_connection", HyperConnectionBlock)

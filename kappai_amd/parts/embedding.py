@@ -44,9 +44,11 @@ class OutputHead(Part):
     table itself (kappai: src/model.c:2562-2571)."""
 
     def __init__(self, name: str, vocab: int, width: int, tied_to: Optional[TokenEmbedding],
-                 suffix: str = ".weight"):
+                 suffix: str = ".weight", softcap: float = 0.0):
+        """``softcap`` c > 0: the logits leave as ``c * tanh(logits / c)``."""
         self.linear = Linear([name], width, [vocab], stage="logits_matmul", weight_suffix=suffix)
         self.tied_to = tied_to
+        self.softcap = float(softcap)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [] if self.tied_to is not None else self.linear.tensor_specs()
@@ -63,7 +65,11 @@ class OutputHead(Part):
     takes_deferred_rows = True     # a plain product: it takes what ops.linear takes
 
     def forward(self, x) -> torch.Tensor:
-        return self.linear.forward(x, out_dtype=torch.float32)
+        logits = self.linear.forward(x, out_dtype=torch.float32)
+        if self.softcap:
+            with profile.scope("logits_matmul"):
+                ops.softcap_rows(logits, self.softcap)
+        return logits
 
     def c_linear(self):
         """The head's product as the C side of a step runs it (float32 logits)."""

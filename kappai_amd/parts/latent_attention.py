@@ -8,7 +8,10 @@ unrotated key ``W_uk[h] c`` and the value ``W_uv[h] c``;
     score(i, j) = (q_un_i . W_uk[h] c_j + q_rot_i . k_rot_j) * scale
 
 over the last ``window`` positions (None: all), a softmax whose denominator may hold
-``exp(sink[h])``, then ``W_o`` on the heads' values side by side.
+``exp(sink[h])``, then ``W_o`` on the heads' values side by side.  ``q_rank``: the queries come
+through a latent of their own, ``q = W_uq n(W_dq h)`` with ``n`` an RMS norm with a weight.
+``gate``: the heads' values side by side are multiplied, channel by channel, by
+``sigmoid(W_g h)`` before ``W_o``.
 
 Only ``c`` and the rotated part are kept per token.  ``q_un . W_uk c = (W_uk^T q_un) . c`` and
 ``sum_j p_j W_uv c_j = W_uv sum_j p_j c_j``: the queries are taken to the latent's space first
@@ -35,10 +38,11 @@ class LatentAttention(Mixer):
     def __init__(self, prefix: str, width: int, num_heads: int, dim: int, rot_dim: int, vdim: int,
                  rank: int, scale: float, norm_eps: float, dtype: torch.dtype,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
-                 sink: bool = False, names=None, weight_suffix: str = ".weight"):
+                 sink: bool = False, names=None, weight_suffix: str = ".weight",
+                 q_rank: Optional[int] = None, gate: bool = False):
         """``position``: a rotary encoding over (part of) the ``rot_dim`` places, or None."""
         n = {"q": "q", "dkv": "dkv", "c_norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o",
-             "sink": "sink"}
+             "sink": "sink", "dq": "dq", "q_norm": "dq.norm", "uq": "uq", "gate": "g"}
         n.update(names or {})
         self.prefix, self.width, self.dtype = prefix, width, dtype
         self.H, self.d, self.rot, self.dv, self.r = num_heads, dim, rot_dim, vdim, rank
@@ -46,9 +50,21 @@ class LatentAttention(Mixer):
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.window = int(window) if window else None
         self.position, self.has_sink = position, sink
-        self.q_dkv = Linear([prefix + n["q"], prefix + n["dkv"]], width,
-                            [num_heads * (dim + rot_dim), rank + rot_dim], stage="matmul_qkv",
-                            weight_suffix=weight_suffix)
+        self.q_rank, self.has_gate = (int(q_rank) if q_rank else None), bool(gate)
+        nq = num_heads * (dim + rot_dim)
+        first, sizes = [prefix + n["q"], prefix + n["dkv"]], [nq, rank + rot_dim]
+        self.up_q = None
+        if self.q_rank:
+            first[0], sizes[0] = prefix + n["dq"], self.q_rank
+            self.up_q = Linear([prefix + n["uq"]], self.q_rank, [nq], stage="matmul_qkv",
+                               weight_suffix=weight_suffix)
+        if self.has_gate:
+            first.append(prefix + n["gate"])
+            sizes.append(num_heads * vdim)
+        self._first_sizes = sizes
+        self.q_dkv = Linear(first, width, sizes, stage="matmul_qkv", weight_suffix=weight_suffix)
+        self._q_norm = prefix + n["q_norm"]
+        self.q_norm_w = None
         self.out = Linear([prefix + n["o"]], num_heads * vdim, [width], stage="matmul_attn_out",
                           weight_suffix=weight_suffix)
         self._uk, self._uv = prefix + n["uk"] + weight_suffix, prefix + n["uv"] + weight_suffix
@@ -72,11 +88,17 @@ class LatentAttention(Mixer):
             TensorSpec(self._c_norm, (self.r,), VECTOR, INIT_ONES)]
         if self.has_sink:
             specs.append(TensorSpec(self._sink, (self.H,), VECTOR, INIT_SMALL))
+        if self.up_q is not None:
+            specs += self.up_q.tensor_specs()
+            specs.append(TensorSpec(self._q_norm, (self.q_rank,), VECTOR, INIT_ONES))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.q_dkv.bind(tensors)
         self.out.bind(tensors)
+        if self.up_q is not None:
+            self.up_q.bind(tensors)
+            self.q_norm_w = tensors[self._q_norm].to(torch.float32).contiguous()
         H, d, dv, r = self.H, self.d, self.dv, self.r
         # [H, out, in] each: to the latent's space (W_uk[h]^T) and from it (W_uv[h])
         self.to_latent = tensors[self._uk].reshape(H, d, r).transpose(1, 2).contiguous()
@@ -90,17 +112,24 @@ class LatentAttention(Mixer):
             raise ValueError("this attention does not read another layer's keys")
         H, d, rot, r, D = self.H, self.d, self.rot, self.r, self.head_size
         proj = self.q_dkv.forward(x)
-        nq = H * (d + rot)
+        nq = self._first_sizes[0]
+        queries = proj
+        if self.up_q is not None:
+            # the queries' own latent: normed in float32, then up to the heads
+            with profile.scope("rope_kvput"):
+                cq = ops.rows_rmsnorm(proj, nq, self.q_norm_w, self.norm_eps)
+            queries = self.up_q.forward(cq)
         rotn = self.position.rotation(x.device, batch.max_position) if self.position else None
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")
         with profile.scope("rope_kvput"):
             q = ops.latent_store(
-                proj[:, :nq], proj[:, nq:], H, d, rot, r, D, self.c_norm_w, self.norm_eps,
+                queries[:, :H * (d + rot)], proj[:, nq:nq + r + rot], H, d, rot, r, D,
+                self.c_norm_w, self.norm_eps,
                 rotn.cos if rotn else None, rotn.sin if rotn else None,
                 rotn.rot_dim if rotn else 0, rotn.mode if rotn else ops.ROT_NONE, k_pool, v_pool,
                 batch.row_pos, batch.row_seg, tables, cache.page_size)
-            ops.headwise_linear(proj, d + rot, self.to_latent, out=q, out_head_stride=D)
+            ops.headwise_linear(queries, d + rot, self.to_latent, out=q, out_head_stride=D)
         with profile.scope("attn"):
             ctx = ops.paged_attention(q, H, 1, D, k_pool, v_pool, batch.row_pos, batch.row_seg,
                                       tables, cache.page_size, self.scale,
@@ -113,11 +142,15 @@ class LatentAttention(Mixer):
                                                                           -1),
                                       mods=self.mods)
             heads = ops.headwise_linear(ctx, D, self.from_latent)
+            if self.has_gate:
+                at = nq + r + rot
+                ops.sigmoid_gate(heads, proj[:, at:at + H * self.dv], 1)
         return self.out.forward(heads, partial_sums=True)
 
     def weight_bytes(self) -> int:
         n = self.to_latent.numel() + self.from_latent.numel()
-        return (self.q_dkv.weight_bytes() + self.out.weight_bytes()
+        up_q = self.up_q.weight_bytes() if self.up_q is not None else 0
+        return (self.q_dkv.weight_bytes() + self.out.weight_bytes() + up_q
                 + n * self.to_latent.element_size())
 
 

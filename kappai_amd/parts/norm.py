@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_ONES, INIT_SMALL, VECTOR, TensorSpec
-from .base import Norm, WeightedTerms, register_part
+from .base import Norm, StreamUpdate, WeightedTerms, register_part
 from .cdesc import FoldDesc
 
 
@@ -89,3 +89,63 @@ class RMSNorm(Norm):
 
 
 register_part("norm", "rmsnorm", RMSNorm)
+
+
+class LayerNorm(Norm):
+    """``(x - mean) / sqrt(var + eps) * w`` without a bias (``var``: the mean of the squared
+    deviations), in float32, in one kernel with the sum that precedes it.  The stream it reads may
+    be kept in several copies [T, copies, width] (``read_streams``): the kernel then first gives
+    the copies the update that is pending (``StreamUpdate``) and normalises their weighted sum."""
+
+    takes_partial_sums = True      # the kernel adds [S, T, width] partial sums itself, in order
+
+    def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype, suffix: str = ""):
+        self.name, self.width, self.eps, self.dtype = name, width, float(eps), dtype
+        self.tensor_name = name + suffix
+        self.weight: Optional[torch.Tensor] = None
+        self._ones = {}
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.tensor_name, (self.width,), VECTOR, INIT_ONES)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.tensor_name].to(torch.float32).contiguous()
+
+    def ones(self, *shape) -> torch.Tensor:
+        """A float32 tensor of ones of this shape on the weight's device (made once)."""
+        if shape not in self._ones:
+            self._ones[shape] = torch.ones(shape, dtype=torch.float32, device=self.weight.device)
+        return self._ones[shape]
+
+    def read_streams(self, streams, in_w, pending: Optional[StreamUpdate] = None, source=None,
+                     rows=None) -> torch.Tensor:
+        """Normalised rows of ``sum_s in_w[s] x_s`` over the copies ``streams`` [T, S, width],
+        after ``pending`` has been applied to them in place.  ``source`` [T, width]: the copies
+        are made here, all equal to it.  ``rows``: only these rows (the copies keep their old
+        values)."""
+        S = streams.shape[1]
+        with profile.scope("rmsnorm" if rows is None else "logits_norm"):
+            return ops.hyper_step(
+                streams, S, self.width, source=source,
+                y=None if pending is None else pending.y,
+                mix=None if pending is None else pending.mix,
+                out_w=None if pending is None else pending.out, in_w=in_w, norm_w=self.weight,
+                eps=self.eps, rows=rows, rows_dtype=self.dtype)
+
+    def add_norm(self, resid, delta, rows=None):
+        """The ``Norm`` contract on one stream [T, width]; or, on a stream in copies [T, S, width]
+        with a pending ``StreamUpdate`` (or None), the norm of the copies' plain sum."""
+        if isinstance(delta, ops.Added):
+            delta = None
+        if resid.dim() == 3:
+            if delta is not None and not isinstance(delta, StreamUpdate):
+                raise ValueError("a stream kept in copies takes its updates as StreamUpdate")
+            return self.read_streams(resid, self.ones(resid.shape[1]), pending=delta, rows=rows)
+        pending = None if delta is None else StreamUpdate(delta, self.ones(1, 1), self.ones(1))
+        return self.read_streams(resid.unsqueeze(1), self.ones(1), pending=pending, rows=rows)
+
+    def weight_bytes(self) -> int:
+        return self.width * 4
+
+
+register_part("norm", "layernorm", LayerNorm)

@@ -13,6 +13,12 @@ than the head size (partial rotation).
 ``f_j / factor * ramp_j + f_j * (1 - ramp_j)``: pairs that turn often within the original context
 keep their frequency, slow ones are slowed by ``factor``, and those between are blended.  Cosine
 and sine are then multiplied by ``0.1 * ln(factor) + 1``.
+
+``wavelength_scaling`` (factor, low, high, original) is another rule for the same end, by the
+pair's wavelength ``l = 2 pi / f``: ``f`` stays where ``l < original / high``, becomes
+``f / factor`` where ``l > original / low``, and between the two is
+``(1 - s) f / factor + s f`` with ``s = (original / l - low) / (high - low)``.  Cosine and sine
+keep their size.
 """
 from __future__ import annotations
 
@@ -38,7 +44,8 @@ class Rotation:
 
 class RotaryEncoding(PositionEncoding):
     def __init__(self, head_dim: int, theta: float, rot_dim: Optional[int] = None,
-                 pairing: str = "half", stretch: Optional[dict] = None):
+                 pairing: str = "half", stretch: Optional[dict] = None,
+                 wavelength_scaling: Optional[dict] = None):
         if pairing not in ("half", "interleaved"):
             raise ValueError(f"pairing must be 'half' or 'interleaved', got {pairing!r}")
         self.head_dim = head_dim
@@ -55,6 +62,15 @@ class RotaryEncoding(PositionEncoding):
                     or self.theta <= 1.0):
                 raise ValueError(f"stretched rotation needs positive numbers and a base above 1, "
                                  f"got {self.stretch} with base {self.theta}")
+        self.wavelength_scaling = None
+        if wavelength_scaling:
+            ws = {k: float(wavelength_scaling[k]) for k in ("factor", "low", "high", "original")}
+            if stretch:
+                raise ValueError("one rule for the frequencies of long contexts, not two")
+            if ws["factor"] <= 0.0 or ws["original"] <= 0.0 or not ws["high"] > ws["low"] > 0.0:
+                raise ValueError(f"scaling by wavelength needs a positive factor and original "
+                                 f"length and high > low > 0, got {ws}")
+            self.wavelength_scaling = ws
         self._rotation: Optional[Rotation] = None
         self._retired = []      # earlier, shorter tables: captured graphs may still read them
 
@@ -62,6 +78,15 @@ class RotaryEncoding(PositionEncoding):
         """(float64 frequencies of the pairs, factor on cosine and sine)."""
         half = self.rot_dim // 2
         freq = np.power(self.theta, -2.0 * np.arange(half, dtype=np.float64) / self.rot_dim)
+        ws = self.wavelength_scaling
+        if ws is not None:
+            wave = 2.0 * math.pi / freq
+            blend = (ws["original"] / wave - ws["low"]) / (ws["high"] - ws["low"])
+            between = (1.0 - blend) * freq / ws["factor"] + blend * freq
+            freq = np.where(wave < ws["original"] / ws["high"], freq,
+                            np.where(wave > ws["original"] / ws["low"], freq / ws["factor"],
+                                     between))
+            return freq, 1.0
         st = self.stretch
         if st is None:
             return freq, 1.0

@@ -12,7 +12,12 @@ softmax whose denominator also holds ``exp(sink[h])``, the weighted sum of the v
 With ``position`` (a rotary encoding) the first places of every q and k head turn by the
 position instead of the norm and the temperature; ``bias``: q, k and v have biases;
 ``values_from_keys``: there is no ``W_v``, a kv head's value is its key as projected, before the
-rotation.  ``bucket``: a distance below half the
+rotation.  ``head_qk_norm``: every q and k head is divided by the root mean square of its own
+``dim`` places and multiplied by a weight of that size which all heads share, before the
+rotation.  ``sink_value``: the sink is this constant score for every head (0: a one in the
+softmax's denominator) and no tensor.  ``head_gate``: a map ``W_g`` [heads, width] of the mixer's
+input gives one number a head, and the head's result is multiplied by its sigmoid before ``W_o``.
+``bucket``: a distance below half the
 table's rows has a row of its own; larger ones share rows on a logarithmic scale that reaches the
 last row at ``bias_max``.  Every piece is optional (``softcap`` 0, no table, no sink, no norm, no
 temperature), so the part also serves designs that use some of them.
@@ -67,9 +72,10 @@ class ScoredAttention(Mixer):
                  temp_coef: float = 0.0, temp_every: int = 1, window: Optional[int] = None,
                  names=None, weight_suffix: str = ".weight", chunk: Optional[int] = None,
                  position=None, bias: bool = False, bias_suffix: str = ".bias",
-                 values_from_keys: bool = False):
+                 values_from_keys: bool = False, head_qk_norm: bool = False,
+                 sink_value: Optional[float] = None, head_gate: bool = False):
         n = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm",
-             "rel": "rel", "sink": "sink"}
+             "rel": "rel", "sink": "sink", "gate": "g"}
         n.update(names or {})
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot be shared out over {num_kv_heads} kv heads")
@@ -88,6 +94,14 @@ class ScoredAttention(Mixer):
         if self.window and self.chunk:
             raise ValueError(f"{prefix}: a sliding window or chunks, not both")
         self.position, self.values_from_keys = position, bool(values_from_keys)
+        self.head_qk_norm, self.head_gate = bool(head_qk_norm), bool(head_gate)
+        self.sink_value = None if sink_value is None else float(sink_value)
+        if self.head_qk_norm and (whole_qk_norm or temp_coef or self.values_from_keys):
+            raise ValueError(f"{prefix}: the norm of every head by itself goes with neither the "
+                             "whole-projection norm, the query temperature nor values that are "
+                             "the keys")
+        if self.sink_value is not None and sink:
+            raise ValueError(f"{prefix}: a learned sink or a constant one, not both")
         if position is not None and (whole_qk_norm or temp_coef):
             raise ValueError(f"{prefix}: a rotation goes with neither the whole-projection norm "
                              "nor the query temperature")
@@ -99,6 +113,10 @@ class ScoredAttention(Mixer):
         stacked = ["q", "k"] + ([] if self.values_from_keys else ["v"])
         sizes = [num_heads * dim, num_kv_heads * dim] + (
             [] if self.values_from_keys else [num_kv_heads * vdim])
+        self._gate_at = sum(sizes)          # where the gates' columns start in the projection
+        if self.head_gate:
+            stacked.append("gate")
+            sizes.append(num_heads)
         self.qkv = Linear([prefix + n[k] for k in stacked], width, sizes, bias=bias,
                           stage="matmul_qkv", weight_suffix=weight_suffix,
                           bias_suffix=bias_suffix)
@@ -124,6 +142,9 @@ class ScoredAttention(Mixer):
         if self.whole_qk_norm:
             specs.append(TensorSpec(self._names["q_norm"], (self.H * self.d,), VECTOR, INIT_ONES))
             specs.append(TensorSpec(self._names["k_norm"], (self.G * self.d,), VECTOR, INIT_ONES))
+        if self.head_qk_norm:
+            specs.append(TensorSpec(self._names["q_norm"], (self.d,), VECTOR, INIT_ONES))
+            specs.append(TensorSpec(self._names["k_norm"], (self.d,), VECTOR, INIT_ONES))
         if self.bias_buckets:
             specs.append(TensorSpec(self._names["rel"], (self.bias_buckets, self.H), VECTOR,
                                     INIT_SMALL))
@@ -142,7 +163,7 @@ class ScoredAttention(Mixer):
             self.out.set_weight(wide.reshape(w.shape[0], H * D).contiguous())
         else:
             self.out.bind(tensors)
-        if self.whole_qk_norm:
+        if self.whole_qk_norm or self.head_qk_norm:
             self.q_norm_w = tensors[self._names["q_norm"]].to(torch.float32).contiguous()
             self.k_norm_w = tensors[self._names["k_norm"]].to(torch.float32).contiguous()
         bias = sink = None
@@ -150,6 +171,9 @@ class ScoredAttention(Mixer):
             bias = distance_bias_columns(tensors[self._names["rel"]], self.bias_far)
         if self.has_sink:
             sink = tensors[self._names["sink"]].to(torch.float32).contiguous()
+        elif self.sink_value is not None:
+            sink = torch.full((H,), self.sink_value, dtype=torch.float32,
+                              device=tensors[self._o_name].device)
         self.mods = ops.ScoreMods(self.softcap, bias, sink)
 
     def forward(self, x, batch, cache, shared_cache: bool = False):
@@ -160,7 +184,15 @@ class ScoredAttention(Mixer):
         tables = batch.block_tables[cache.group]
         k_pool, v_pool = cache.pool("k"), cache.pool("v")
         with profile.scope("rope_kvput"):
-            if self.position is not None or self.values_from_keys:
+            if self.head_qk_norm:
+                rot = (self.position.rotation(x.device, batch.max_position)
+                       if self.position is not None else None)
+                q = ops.head_norm_rotate_store(
+                    proj, H, G, self.d, self.dv, D, self.q_norm_w, self.k_norm_w, self.norm_eps,
+                    rot.cos if rot else None, rot.sin if rot else None,
+                    rot.rot_dim if rot else 0, rot.mode if rot else ops.ROT_NONE, k_pool, v_pool,
+                    batch.row_pos, batch.row_seg, tables, cache.page_size)
+            elif self.position is not None or self.values_from_keys:
                 rot = (self.position.rotation(x.device, batch.max_position)
                        if self.position is not None else None)
                 q = ops.rotate_widen_store(
@@ -184,6 +216,9 @@ class ScoredAttention(Mixer):
                                       max_lone_position=batch.numbers.get("max_lone_position",
                                                                           -1),
                                       mods=self.mods)
+            if self.head_gate:
+                at = self._gate_at
+                ops.sigmoid_gate(ctx, proj[:, at:at + H], D)
         return self.out.forward(ctx, partial_sums=True)
 
     def weight_bytes(self) -> int:

@@ -14,7 +14,7 @@ import numpy as np
 import torch
 
 from .safetensors_io import write_safetensors
-from .spec import INIT_NORMAL, INIT_ONES, INIT_SMALL, TensorSpec
+from .spec import INIT_CONNECT, INIT_NORMAL, INIT_ONES, INIT_SMALL, TensorSpec
 
 
 def _generator(seed: int, name: str) -> np.random.Generator:
@@ -33,6 +33,12 @@ def random_tensor(spec: TensorSpec, seed: int, std: float, norm_jitter: float,
             a += rng.standard_normal(spec.shape, dtype=np.float32) * np.float32(norm_jitter)
     elif spec.init in (INIT_NORMAL, INIT_SMALL):
         a = rng.standard_normal(spec.shape, dtype=np.float32) * np.float32(std)
+    elif spec.init == INIT_CONNECT:
+        noise = rng.standard_normal(spec.shape, dtype=np.float32)
+        if len(spec.shape) == 2 and spec.shape[0] == spec.shape[1]:
+            a = np.eye(spec.shape[0], dtype=np.float32) + np.float32(0.15) * noise
+        else:
+            a = np.float32(0.6) + np.float32(0.25) * noise
     else:
         raise ValueError(f"unknown init {spec.init!r} for {spec.name}")
     t = torch.from_numpy(a)

@@ -14,6 +14,8 @@ TABLE = "table"      # rows looked up by integer id (embeddings); compute dtype
 INIT_NORMAL = "normal"             # N(0, matrix_std)
 INIT_ONES = "ones"                 # 1, or 1 + N(0, norm_jitter) when jitter is asked for
 INIT_SMALL = "small"               # N(0, matrix_std), for biases
+INIT_CONNECT = "connect"           # weights among copies of a stream: a square matrix is the
+                                   # identity + N(0, 0.15), a vector 0.6 + N(0, 0.25)
 
 
 @dataclass(frozen=True)

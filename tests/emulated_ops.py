@@ -677,8 +677,10 @@ class _Plan:
         self.experts = experts
 
 
-def moe_route(x, router, top):
+def moe_route(x, router, top, bias=None):
     logits = x.to(F32) @ router.T
+    if bias is not None:
+        logits = logits + bias
     best, chosen = torch.topk(logits, top, dim=-1)
     return chosen.to(torch.int32), torch.softmax(best, dim=-1)
 
@@ -708,11 +710,95 @@ def moe_experts_down(act, w_down, plan):
     return out
 
 
-def moe_combine(y, weights, plan):
-    return (y * weights[:, :, None]).sum(dim=1)
+def moe_experts_activated(x, w_up, plan):
+    T, top = plan.experts.shape
+    out = torch.empty((T, top, w_up.shape[1]), dtype=x.dtype)
+    for t in range(T):
+        for k in range(top):
+            u = torch.relu(w_up[int(plan.experts[t, k])].to(F32) @ x[t].to(F32))
+            out[t, k] = (u * u).to(x.dtype)
+    return out
 
 
-ALL = ["add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
+def moe_combine(y, weights, plan, also=None):
+    out = (y * weights[:, :, None]).sum(dim=1)
+    if also is not None:
+        for p in (also if also.dim() == 3 else also[None]):
+            out = out + p.to(F32)
+    return out
+
+
+def head_norm_rotate_store(proj, n_heads, n_kv_heads, dim, vdim, head_size, q_norm_w, k_norm_w,
+                           eps, cos, sin, rot_dims, rot_mode, k_pool, v_pool, row_pos, row_seg,
+                           block_tables, page_size):
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    T = proj.shape[0]
+    p = proj.to(F32)
+    pos = row_pos.long()
+    q = p[:, :H * d].reshape(T, H, d)
+    k = p[:, H * d:(H + G) * d].reshape(T, G, d)
+    v = p[:, (H + G) * d:(H + G) * d + G * dv].reshape(T, G, dv)
+    if q_norm_w is not None:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_norm_w
+    if k_norm_w is not None:
+        k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_norm_w
+    qo, ko, vo = (torch.zeros((T, n, D), dtype=F32) for n in (H, G, G))
+    qo[:, :, :d] = _rotate(q, pos, cos, sin, rot_dims, rot_mode)
+    ko[:, :, :d] = _rotate(k, pos, cos, sin, rot_dims, rot_mode)
+    vo[:, :, :dv] = v
+    _store(k_pool, v_pool, ko, vo, row_pos, row_seg, block_tables, page_size)
+    return qo.reshape(T, H * D).to(proj.dtype)
+
+
+HYPER_MAX_STREAMS = 8
+ACT_RELU_SQUARED = 0
+
+
+def hyper_step(streams, n_streams, width, source=None, y=None, mix=None, out_w=None, in_w=None,
+               norm_w=None, eps=0.0, rows=None, rows_dtype=None, store=True):
+    S = n_streams
+    x = source[:, None, :].expand(-1, S, -1).to(F32) if source is not None else streams
+    new = x
+    if y is not None:
+        upd = torch.zeros_like(x[:, 0])
+        for p in (y if y.dim() == 3 else y[None]):
+            upd = upd + p.to(F32)
+        new = torch.einsum("st,nsw->ntw", mix, x) + out_w[None, :, None] * upd[:, None, :]
+    if rows is None and store and streams is not None and (y is not None or source is not None):
+        streams.copy_(new)
+    if rows_dtype is None:
+        return None
+    u = torch.einsum("s,nsw->nw", in_w, new)
+    if rows is not None:
+        u = u[rows.long()]
+    dev = u - u.mean(-1, keepdim=True)
+    return (dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + eps) * norm_w).to(rows_dtype)
+
+
+def rows_rmsnorm(x, n, weight, eps):
+    v = x[:, :n].to(F32)
+    return (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight).to(x.dtype)
+
+
+def sigmoid_gate(x, gate, group):
+    T, n = x.shape
+    g = torch.sigmoid(gate[:, :n // group].to(F32)).repeat_interleave(group, dim=1)
+    x.copy_((x.to(F32) * g).to(x.dtype))
+    return x
+
+
+def softcap_rows(x, cap):
+    x.copy_(cap * torch.tanh(x / cap))
+    return x
+
+
+def activate(x, kind=0):
+    r = torch.relu(x.to(F32))
+    return (r * r).to(x.dtype)
+
+
+ALL = ["moe_experts_activated", "head_norm_rotate_store", "hyper_step", "rows_rmsnorm", "sigmoid_gate",
+       "softcap_rows", "activate", "add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
        "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
        "output_norm_add", "projection_norm_store", "latent_store", "headwise_linear", "conv_silu",
        "matrix_state_recurrence", "head_norm_gate", "rotate_widen_store", "token_shift_mix", "tanh",
