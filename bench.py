@@ -112,7 +112,12 @@ COMPARISONS = {"w1024": ("dapipel-w1024", "lfm2-like-w1024"),
                # the Zumuzen decoder beside them as well (pairs of mixers where the LFM2 shapes
                # have attention, a gated recurrence per channel where they have convolutions)
                "zumuzen-w1024": ("zumuzen-w1024", "lfm2-like-w1024"),
-               "zumuzen-w2048": ("zumuzen-w2048", "lfm2-like-w2048")}
+               "zumuzen-w2048": ("zumuzen-w2048", "lfm2-like-w2048"),
+               # the Sibodra decoder beside the Dukolorn decoder of equal size (its closest
+               # relative: the same two attention parts, scores worked on before the softmax, a
+               # latent for keys and values) and beside the same LFM2 shapes
+               "sibodra-w1024": ("sibodra-w1024", "dukolorn-w1024", "lfm2-like-w1024"),
+               "sibodra-w2048": ("sibodra-w2048", "dukolorn-w2048", "lfm2-like-w2048")}
 
 
 def stage_table(runner, entries_of, reps):
@@ -194,10 +199,9 @@ def measure_model(name, dtype, device, prefill_tokens, batch, context, steps, wa
 def run_comparison(keys, args):
     results = {}
     for key in keys:
-        new, old = COMPARISONS[key]
         results[key] = [measure_model(n, args.dtype, "cuda:0", args.prefill_tokens, args.batch,
                                       min(args.context, 2048), args.steps, args.warmup,
-                                      args.page_size) for n in (new, old)]
+                                      args.page_size) for n in COMPARISONS[key]]
         print(f"bench.py: {key} done", file=sys.stderr, flush=True)
     print(json.dumps({"metric": "prefill and decode tok/s, a decoder beside the LFM2 shape of "
                                 "equal size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
@@ -572,13 +576,13 @@ def main() -> int:
                          "the greedy choice (1: none)")
     ap.add_argument("--compare", default="", metavar="SIZES",
                     help="instead of the headline run: prompt and decode steps of the Dapipel, "
-                         "Dukolorn or Zumuzen decoder beside the LFM2 shape of equal size, at these sizes (comma "
+                         "Dukolorn, Zumuzen or Sibodra decoder beside the LFM2 shape of equal size, at these sizes (comma "
                          "separated: " + ", ".join(sorted(COMPARISONS)) + "; 'all')")
     args = ap.parse_args()
     if args.compare:
         keys = (sorted(k for k in COMPARISONS if k.startswith("w")) if args.compare == "all"
                 else sorted(k for k in COMPARISONS if k.startswith(args.compare + "-"))
-                if args.compare in ("dukolorn", "zumuzen") else args.compare.split(","))
+                if args.compare in ("dukolorn", "zumuzen", "sibodra") else args.compare.split(","))
         for k in keys:
             if k not in COMPARISONS:
                 print(f"bench.py: no comparison {k!r}; known: {', '.join(sorted(COMPARISONS))}")

@@ -199,6 +199,50 @@ SHAPES.update({
 })
 
 
+def _sibodra(width, mixers, heads, kv_heads, dim, rot, l_heads, l_dim, l_rot, l_vdim, l_rank,
+             q_rank, ff, experts, top, streams, vocab=65536, original=8192) -> dict:
+    """Layers by letter: "a" grouped-query attention (per-head norms, partial rotation with scaled
+    frequencies, capped scores), "l" latent attention; dense feed-forwards of ``ff`` and mixtures
+    of ``experts`` squared-ReLU experts of ``ff // top`` with a shared expert of the same size in
+    turns; the stream in ``streams`` copies."""
+    layers = []
+    for i, kind in enumerate(mixers):
+        if kind == "a":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                     "scale": dim ** -0.5, "softcap": 50.0,
+                     "rot": {"base": 10000.0, "dims": rot,
+                             "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                         "original": original}}}
+        else:
+            mixer = {"heads": l_heads, "dim": l_dim, "rot_dim": l_rot, "vdim": l_vdim,
+                     "kv_rank": l_rank, "q_rank": q_rank, "scale": (l_dim + l_rot) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": l_rot}}
+        mlp = ({"kind": "dense", "ff": ff} if i % 2 == 0 else
+               {"kind": "moe", "expert": {"ff": ff // top}, "shared": {"ff": ff // top},
+                "router": {"experts": experts, "top": top}})
+        layers.append({"type": "attention" if kind == "a" else "latent_attention",
+                       "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Sibodra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "streams": streams, "logit_softcap": 30.0, "layers": layers}
+
+
+SHAPES.update({
+    # eight layers at a width of 1024, grouped-query and latent attention in turns: 16 heads of
+    # 64 on 4 kv heads, half of every head rotated; 16 latent heads of 64 + 32 rotated places on
+    # a latent of 224, queries through a latent of 384; feed-forward 4608 dense or 16 experts of
+    # 2304 beside a shared one, two a token; the stream in four copies
+    "sibodra-w1024": _sibodra(1024, "alalalal", 16, 4, 64, 32, 16, 64, 32, 64, 224, 384, 4608,
+                              16, 2, 4),
+    # the same at a width of 2048: 32 heads on 8 kv heads, 16 latent heads of 128 + 64 on a
+    # latent of 192, queries through a latent of 768, feed-forward 8192
+    "sibodra-w2048": _sibodra(2048, "alalalal", 32, 8, 64, 32, 16, 128, 64, 128, 192, 768, 8192,
+                              16, 2, 4),
+    # a tiny one for smoke runs
+    "sibodra-tiny": _sibodra(64, "ala", 4, 2, 8, 4, 2, 8, 8, 16, 24, 16, 96, 4, 2, 2, vocab=256,
+                             original=64),
+})
+
+
 def named_shape(name: str) -> dict:
     """A copy of the configuration called ``name`` (any case), or a ``KeyError`` naming them all."""
     key = name.strip().lower()
