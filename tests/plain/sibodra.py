@@ -162,9 +162,15 @@ def expert(h, t, p: str, rounding=None):
     return matmul(z * z, t[p + "down"], rounding)
 
 
-def moe_ff(h, t, p: str, mlp: dict, rounding=None):
+def moe_ff(h, t, p: str, mlp: dict, rounding=None, margins: list = None):
+    """``margins``: gets, row by row, how far the last chosen logit stands above the first one
+    that was not chosen (infinite when every expert is chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     logits = _r(h, rounding) @ t[p + "router"].to(F64).T + t[p + "router.b"].to(F64)
+    if margins is not None:
+        srt = logits.sort(dim=1, descending=True).values
+        margins.append(srt[:, top - 1] - srt[:, top] if top < E
+                       else torch.full((h.shape[0],), math.inf, dtype=F64))
     out = torch.zeros_like(h)
     for i in range(h.shape[0]):
         order = sorted(range(E), key=lambda e: (-float(logits[i, e]), e))[:top]
@@ -178,9 +184,9 @@ def moe_ff(h, t, p: str, mlp: dict, rounding=None):
 
 
 def forward(cfg: dict, t: Dict[str, torch.Tensor], tokens: List[int], rounding=None,
-            layers_out: list = None):
+            layers_out: list = None, margins: list = None):
     """Float64 logits [len(tokens), vocab].  ``layers_out``: gets the sum of the stream's copies
-    after every layer."""
+    after every layer; ``margins``: gets every router's margins (``moe_ff``)."""
     eps = cfg["norm"]["eps"]
     S = cfg.get("streams")
     x = t["embed"].to(F64)[torch.tensor(tokens, dtype=torch.long)]
@@ -211,7 +217,7 @@ def forward(cfg: dict, t: Dict[str, torch.Tensor], tokens: List[int], rounding=N
             if mlp["kind"] == "dense":
                 sublayer(2, p, lambda h: dense_ff(h, t, p + "mlp.", rounding))
             else:
-                sublayer(2, p, lambda h: moe_ff(h, t, p + "mlp.", mlp, rounding))
+                sublayer(2, p, lambda h: moe_ff(h, t, p + "mlp.", mlp, rounding, margins))
         if layers_out is not None:
             layers_out.append(sum(xs))
     x = layer_norm(sum(xs), t["final.norm"], eps)

@@ -445,13 +445,17 @@ def test_schedules(tmp_path, model_dirs, name, family, dtype):
 def test_long_decoding(tmp_path, model_dirs, dtype):
     """A short prompt and 330 tokens one by one (pages taken one after the other, the block tables
     of a graph grown, the rotation tables grown past their first size), two requests side by
-    side."""
-    for name in ("A", "D"):
+    side.  In bfloat16 the configuration whose routers choose every expert is held to the plain
+    implementation row by row to the end; the others meet a router's close call early, from where
+    on their rows must stay finite and of the logits' size (their float32 runs are held to every
+    row)."""
+    for name in ("A", "B", "D"):
         requests = make_requests(TINY[name][0]["vocab"], [350, 290], seed=22)
         plans = {"r0": (0, [20] + [1] * 330), "r1": (5, [3] + [1] * 287)}
         steps, index, peak = schedules.build(requests, plans)
         got, runner = replay(model_dirs[name], dtype, steps, index, peak, tmp_path / name)
-        assert_matches_plain(got, model_dirs[name], requests, dtype, (name, dtype))
+        assert_matches_plain(got, model_dirs[name], requests, dtype, (name, dtype),
+                             min_strict=1.0 if name == "B" else 0.0)
         assert runner.graph_replays > 250
 
 
