@@ -172,7 +172,9 @@ extern "C" int kappai_latent_store(const void* q, int q_stride, const void* kv, 
 // ---------------------------------------------------------------------------------------
 // y[t, h, o] = sum_i W[h, o, i] x[t, h, i]: W [H, n_out, n_in] in the activations' dtype, x and y
 // with a row stride and a head stride each, float accumulation.  A block takes 32 rows x 64
-// outputs of one head; x and W tiles go through LDS in steps of 32 along i.
+// outputs of one head; x and W tiles go through LDS in steps of 32 along i.  With `gate` (rows
+// of stride g_row, column h n_out + o) the result is multiplied by sigmoid(gate) before it is
+// stored.
 // ---------------------------------------------------------------------------------------
 #define HW_BM 32
 #define HW_BN 64
@@ -181,7 +183,7 @@ extern "C" int kappai_latent_store(const void* q, int q_stride, const void* kv, 
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(
     const T* __restrict__ x, int x_row, int x_head, const T* __restrict__ w, int n_out, int n_in,
-    TO* __restrict__ y, int y_row, int y_head, int rows) {
+    TO* __restrict__ y, int y_row, int y_head, int rows, const T* __restrict__ gate, int g_row) {
   __shared__ float xs[HW_BM][HW_BK + 1];
   __shared__ float ws[HW_BN][HW_BK + 1];
   const int h = blockIdx.z, m0 = blockIdx.x * HW_BM, n0 = blockIdx.y * HW_BN;
@@ -220,7 +222,10 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + 4 * tx + j;
-      if (n < n_out) from_f32(y + (size_t)m * y_row + (size_t)h * y_head + n, acc[i][j]);
+      if (n >= n_out) continue;
+      float v = acc[i][j];
+      if (gate) v /= 1.0f + expf(-to_f32(gate[(size_t)m * g_row + (size_t)h * n_out + n]));
+      from_f32(y + (size_t)m * y_row + (size_t)h * y_head + n, v);
     }
   }
 }
@@ -237,7 +242,8 @@ typedef __attribute__((ext_vector_type(4))) float hw_f32x4_t;
 template <typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
     const bf16_t* __restrict__ x, int x_row, int x_head, const bf16_t* __restrict__ w, int n_out,
-    int n_in, TO* __restrict__ y, int y_row, int y_head, int rows) {
+    int n_in, TO* __restrict__ y, int y_row, int y_head, int rows,
+    const bf16_t* __restrict__ gate, int g_row) {
   const int h = blockIdx.z, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int m0 = (blockIdx.x * (blockDim.x / WAVE) + wave) * 16, n0 = blockIdx.y * 64;
   if (m0 >= rows) return;
@@ -271,14 +277,19 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int n = n0 + 16 * j + 4 * kq + v;
-      if (n < n_out) from_f32(yr + n, acc[j][v]);
+      if (n >= n_out) continue;
+      float r = acc[j][v];
+      if (gate)
+        r /= 1.0f + expf(-bf16_to_f32(gate[(size_t)(m0 + lr) * g_row + (size_t)h * n_out + n]));
+      from_f32(yr + n, r);
     }
 }
 
 // out_f32: the results stay float32 although x and W are bfloat16 (what enters a recurrence).
 extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, const void* w, int H,
                                       int n_out, int n_in, void* y, int y_row, int y_head,
-                                      int rows, int is_bf16, int out_f32, hipStream_t stream) {
+                                      int rows, int is_bf16, int out_f32, const void* gate,
+                                      int g_row, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H < 1 || H > 65535 || n_out < 1 || n_in < 1) return (int)hipErrorInvalidValue;
   if (is_bf16 && n_in % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 &&
@@ -288,11 +299,11 @@ extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, cons
     if (out_f32)
       hipLaunchKernelGGL(headwise_linear_mfma_kernel<float>, grid, dim3(waves * WAVE), 0, stream,
                          (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in,
-                         (float*)y, y_row, y_head, rows);
+                         (float*)y, y_row, y_head, rows, (const bf16_t*)gate, g_row);
     else
       hipLaunchKernelGGL(headwise_linear_mfma_kernel<bf16_t>, grid, dim3(waves * WAVE), 0, stream,
                          (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in,
-                         (bf16_t*)y, y_row, y_head, rows);
+                         (bf16_t*)y, y_row, y_head, rows, (const bf16_t*)gate, g_row);
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
   dim3 grid((rows + HW_BM - 1) / HW_BM, (n_out + HW_BN - 1) / HW_BN, H);
@@ -300,15 +311,15 @@ extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, cons
   if (is_bf16 && out_f32)
     hipLaunchKernelGGL((headwise_linear_kernel<bf16_t, float>), grid, dim3(256), 0, stream,
                        (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in, (float*)y,
-                       y_row, y_head, rows);
+                       y_row, y_head, rows, (const bf16_t*)gate, g_row);
   else if (is_bf16)
     hipLaunchKernelGGL((headwise_linear_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream,
                        (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in, (bf16_t*)y,
-                       y_row, y_head, rows);
+                       y_row, y_head, rows, (const bf16_t*)gate, g_row);
   else
     hipLaunchKernelGGL((headwise_linear_kernel<float, float>), grid, dim3(256), 0, stream,
                        (const float*)x, x_row, x_head, (const float*)w, n_out, n_in, (float*)y,
-                       y_row, y_head, rows);
+                       y_row, y_head, rows, (const float*)gate, g_row);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

@@ -17,16 +17,67 @@
 #define HS_THREADS 256
 #define HS_MAX_STREAMS 8
 
-// y of row t, column c: rows of TY, or P float planes [P, T, W] added in order
-template <typename TY>
-__device__ __forceinline__ float update_at(const TY* __restrict__ y, int parts, size_t plane,
-                                           size_t at) {
-  float v = to_f32(y[at]);
-  for (int p = 1; p < parts; ++p) v += to_f32(y[(size_t)p * plane + at]);
-  return v;
+// VEC values of an update from column c on: rows of TY, or P float planes [P, T, W] added in order
+template <int VEC>
+__device__ __forceinline__ void update_at(const float* __restrict__ y, int parts, size_t plane,
+                                          size_t at, float* v) {
+  if (VEC == 4) {
+    const float4 a = *reinterpret_cast<const float4*>(y + at);
+    v[0] = a.x; v[VEC > 1 ? 1 : 0] = a.y; v[VEC > 2 ? 2 : 0] = a.z; v[VEC > 3 ? 3 : 0] = a.w;
+    for (int p = 1; p < parts; ++p) {
+      const float4 b = *reinterpret_cast<const float4*>(y + (size_t)p * plane + at);
+      v[0] += b.x; v[VEC > 1 ? 1 : 0] += b.y; v[VEC > 2 ? 2 : 0] += b.z; v[VEC > 3 ? 3 : 0] += b.w;
+    }
+  } else {
+    v[0] = y[at];
+    for (int p = 1; p < parts; ++p) v[0] += y[(size_t)p * plane + at];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void update_at(const bf16_t* __restrict__ y, int, size_t, size_t at,
+                                          float* v) {
+  if (VEC == 4) {
+    const uint2 a = *reinterpret_cast<const uint2*>(y + at);
+    v[0] = __uint_as_float(a.x << 16);
+    v[VEC > 1 ? 1 : 0] = __uint_as_float(a.x & 0xffff0000u);
+    v[VEC > 2 ? 2 : 0] = __uint_as_float(a.y << 16);
+    v[VEC > 3 ? 3 : 0] = __uint_as_float(a.y & 0xffff0000u);
+  } else {
+    v[0] = bf16_to_f32(y[at]);
+  }
 }
 
-template <typename TY, typename TO>
+template <int VEC>
+__device__ __forceinline__ void load_f32(const float* p, float* v) {
+  if (VEC == 4) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[VEC > 1 ? 1 : 0] = a.y; v[VEC > 2 ? 2 : 0] = a.z; v[VEC > 3 ? 3 : 0] = a.w;
+  } else {
+    v[0] = p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void store_f32(float* p, const float* v) {
+  if (VEC == 4)
+    *reinterpret_cast<float4*>(p) =
+        make_float4(v[0], v[VEC > 1 ? 1 : 0], v[VEC > 2 ? 2 : 0], v[VEC > 3 ? 3 : 0]);
+  else
+    p[0] = v[0];
+}
+template <int VEC>
+__device__ __forceinline__ void store_rows(float* p, const float* v) { store_f32<VEC>(p, v); }
+template <int VEC>
+__device__ __forceinline__ void store_rows(bf16_t* p, const float* v) {
+  if (VEC == 4)
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v[0], v[VEC > 1 ? 1 : 0]),
+                                              pack_bf16x2(v[VEC > 2 ? 2 : 0], v[VEC > 3 ? 3 : 0]));
+  else
+    p[0] = f32_to_bf16(v[0]);
+}
+
+// A block a row; a thread takes VEC neighbouring columns at a time (VEC 4: 16-byte loads and
+// stores; the width and every address then are multiples of four values).
+template <typename TY, typename TO, int VEC>
 __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
     float* __restrict__ streams, const float* __restrict__ source, const TY* __restrict__ y,
     int parts, const float* __restrict__ mix, const float* __restrict__ out_w,
@@ -46,54 +97,72 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   const bool write = y != nullptr, read = normed != nullptr;
   const size_t plane = (size_t)T * W;
   float sum = 0.f;
-  for (int c = tid; c < W; c += HS_THREADS) {
-    float x[HS_MAX_STREAMS];
+  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+    float x[HS_MAX_STREAMS][VEC];
 #pragma unroll
     for (int s = 0; s < HS_MAX_STREAMS; ++s)
-      if (s < S) x[s] = source ? source[(size_t)t * W + c] : streams[((size_t)t * S + s) * W + c];
+      if (s < S)
+        load_f32<VEC>(source ? source + (size_t)t * W + c : streams + ((size_t)t * S + s) * W + c,
+                      x[s]);
     if (write) {
-      const float yv = update_at(y, parts, plane, (size_t)t * W + c);
-      float nx[HS_MAX_STREAMS];
+      float yv[VEC];
+      update_at<VEC>(y, parts, plane, (size_t)t * W + c, yv);
+      float nx[HS_MAX_STREAMS][VEC];
 #pragma unroll
       for (int to = 0; to < HS_MAX_STREAMS; ++to)
         if (to < S) {
-          float acc = 0.f;
 #pragma unroll
-          for (int s = 0; s < HS_MAX_STREAMS; ++s)
-            if (s < S) acc = fmaf(c_mix[s * S + to], x[s], acc);
-          nx[to] = fmaf(c_out[to], yv, acc);
+          for (int i = 0; i < VEC; ++i) {
+            float acc = 0.f;
+#pragma unroll
+            for (int s = 0; s < HS_MAX_STREAMS; ++s)
+              if (s < S) acc = fmaf(c_mix[s * S + to], x[s][i], acc);
+            nx[to][i] = fmaf(c_out[to], yv[i], acc);
+          }
         }
 #pragma unroll
       for (int s = 0; s < HS_MAX_STREAMS; ++s)
         if (s < S) {
-          x[s] = nx[s];
-          if (store) streams[((size_t)t * S + s) * W + c] = nx[s];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) x[s][i] = nx[s][i];
+          if (store) store_f32<VEC>(streams + ((size_t)t * S + s) * W + c, nx[s]);
         }
     } else if (source && store) {
 #pragma unroll
       for (int s = 0; s < HS_MAX_STREAMS; ++s)
-        if (s < S) streams[((size_t)t * S + s) * W + c] = x[s];
+        if (s < S) store_f32<VEC>(streams + ((size_t)t * S + s) * W + c, x[s]);
     }
     if (read) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < HS_MAX_STREAMS; ++s)
-        if (s < S) u = fmaf(c_in[s], x[s], u);
-      u_row[c] = u;
-      sum += u;
+      for (int i = 0; i < VEC; ++i) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < HS_MAX_STREAMS; ++s)
+          if (s < S) u = fmaf(c_in[s], x[s][i], u);
+        u_row[c + i] = u;
+        sum += u;
+      }
     }
   }
   if (!read) return;
   const float mean = block_sum(sum, red) / (float)W;
   float sq = 0.f;
-  for (int c = tid; c < W; c += HS_THREADS) {
-    const float d = u_row[c] - mean;
-    sq = fmaf(d, d, sq);
+  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float d = u_row[c + i] - mean;
+      sq = fmaf(d, d, sq);
+    }
   }
   const float rstd = 1.0f / sqrtf(block_sum(sq, red) / (float)W + eps);
   TO* dst = normed + (size_t)blockIdx.x * W;
-  for (int c = tid; c < W; c += HS_THREADS)
-    from_f32(dst + c, (u_row[c] - mean) * rstd * norm_w[c]);
+  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+    float o[VEC], w[VEC];
+    load_f32<VEC>(norm_w + c, w);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = (u_row[c + i] - mean) * rstd * w[i];
+    store_rows<VEC>(dst + c, o);
+  }
 }
 
 extern "C" int kappai_hyper_step(float* streams, const float* source, const void* y,
@@ -109,16 +178,21 @@ extern "C" int kappai_hyper_step(float* streams, const float* source, const void
     return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)(W + 16) * sizeof(float);
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
-#define HS_LAUNCH(TY, TO)                                                                        \
-  hipLaunchKernelGGL((hyper_step_kernel<TY, TO>), dim3(blocks), dim3(HS_THREADS), lds, stream,   \
+  const bool vec = W % 4 == 0 && ((uintptr_t)streams | (uintptr_t)source | (uintptr_t)norm_w |
+                                  (uintptr_t)normed) % 16 == 0 && (uintptr_t)y % 16 == 0;
+#define HS_LAUNCH_V(TY, TO, V)                                                                   \
+  hipLaunchKernelGGL((hyper_step_kernel<TY, TO, V>), dim3(blocks), dim3(HS_THREADS), lds, stream, \
                      streams, source, (const TY*)y, parts, mix, out_w, in_w, norm_w, eps, rows,   \
                      store, (TO*)normed, T, S, W)
+#define HS_LAUNCH(TY, TO)                                                                        \
+  if (vec) HS_LAUNCH_V(TY, TO, 4); else HS_LAUNCH_V(TY, TO, 1)
   if (y_is_bf16) {
-    if (normed_is_bf16) HS_LAUNCH(bf16_t, bf16_t); else HS_LAUNCH(bf16_t, float);
+    if (normed_is_bf16) { HS_LAUNCH(bf16_t, bf16_t); } else { HS_LAUNCH(bf16_t, float); }
   } else {
-    if (normed_is_bf16) HS_LAUNCH(float, bf16_t); else HS_LAUNCH(float, float);
+    if (normed_is_bf16) { HS_LAUNCH(float, bf16_t); } else { HS_LAUNCH(float, float); }
   }
 #undef HS_LAUNCH
+#undef HS_LAUNCH_V
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

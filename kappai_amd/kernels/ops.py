@@ -2047,10 +2047,12 @@ def latent_store(q: torch.Tensor, kv: torch.Tensor, n_heads: int, dim: int, rot_
 
 def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor,
                     out: Optional[torch.Tensor] = None, out_head_stride: Optional[int] = None,
-                    out_dtype=None) -> torch.Tensor:
+                    out_dtype=None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``y[t, h, :] = weight[h] @ x[t, h, :]`` with ``weight`` [H, n_out, n_in] in the dtype of
     ``x``.  ``out_dtype`` float32 keeps the sums as they are (else they are stored as ``x`` is).  Head h of row t starts at ``x[t, h * x_head_stride]`` and is written at
-    ``out[t, h * out_head_stride]`` (``out`` None: a new [T, H n_out])."""
+    ``out[t, h * out_head_stride]`` (``out`` None: a new [T, H n_out]).  ``gate`` [T, H n_out] in
+    the dtype of ``x`` (rows may be strided): every result is multiplied by the sigmoid of its
+    gate before it is stored."""
     _gpu("x", x, (F32, BF16), contiguous=False)
     _gpu("weight", weight, x.dtype)
     _need(weight.dim() == 3, "headwise_linear: weight must be [heads, out, in]")
@@ -2068,11 +2070,15 @@ def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor,
     _need(out.dim() == 2 and out.shape[0] == T and out.stride(1) == 1
           and (H - 1) * out_head_stride + n_out <= out.shape[1],
           lambda: f"headwise_linear: out {tuple(out.shape)}")
+    if gate is not None:
+        _gpu("gate", gate, x.dtype, contiguous=False)
+        _need(gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H * n_out
+              and gate.stride(1) == 1, lambda: f"headwise_linear: gate {tuple(gate.shape)}")
     check(library("attn_prep").kappai_headwise_linear(
         _ptr(x), _c_int(x.stride(0)), _c_int(x_head_stride), _ptr(weight), _c_int(H),
         _c_int(n_out), _c_int(n_in), _ptr(out), _c_int(out.stride(0)), _c_int(out_head_stride),
-        _c_int(T), _c_int(_is_bf16(x.dtype)), _c_int(1 if out_dtype == F32 else 0), _stream()),
-        "headwise_linear")
+        _c_int(T), _c_int(_is_bf16(x.dtype)), _c_int(1 if out_dtype == F32 else 0), _ptr(gate),
+        _c_int(gate.stride(0) if gate is not None else 0), _stream()), "headwise_linear")
     return out
 
 

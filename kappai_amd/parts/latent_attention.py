@@ -141,10 +141,10 @@ class LatentAttention(Mixer):
                                       max_lone_position=batch.numbers.get("max_lone_position",
                                                                           -1),
                                       mods=self.mods)
-            heads = ops.headwise_linear(ctx, D, self.from_latent)
-            if self.has_gate:
-                at = nq + r + rot
-                ops.sigmoid_gate(heads, proj[:, at:at + H * self.dv], 1)
+            at = nq + r + rot
+            heads = ops.headwise_linear(
+                ctx, D, self.from_latent,
+                gate=proj[:, at:at + H * self.dv] if self.has_gate else None)
         return self.out.forward(heads, partial_sums=True)
 
     def weight_bytes(self) -> int:

@@ -474,7 +474,8 @@ def latent_store(q, kv, n_heads, dim, rot_dim, rank, head_size, c_norm_w, eps, c
     return out.reshape(T, H * D).to(q.dtype)
 
 
-def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None, out_dtype=None):
+def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None, out_dtype=None,
+                    gate=None):
     H, n_out, n_in = weight.shape
     T = x.shape[0]
     if out is None:
@@ -482,8 +483,10 @@ def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None, ou
         out_head_stride = n_out
     for h in range(H):
         xi = x[:, h * x_head_stride:h * x_head_stride + n_in].to(F32)
-        out[:, h * out_head_stride:h * out_head_stride + n_out] = (
-            xi @ weight[h].to(F32).T).to(out.dtype)
+        y = xi @ weight[h].to(F32).T
+        if gate is not None:
+            y = y * torch.sigmoid(gate[:, h * n_out:(h + 1) * n_out].to(F32))
+        out[:, h * out_head_stride:h * out_head_stride + n_out] = y.to(out.dtype)
     return out
 
 
