@@ -402,7 +402,8 @@ extern "C" int kappai_rotate_widen_store(
 // multiplied by a weight [d] that all heads share (q_norm_w / k_norm_w; null: no norm); then the
 // first rot_dims places of the head turn by the row's position.  proj [T, H d + G d + G dv].
 // Queries leave as H heads of D (zeros behind d); keys and values go to the pools as G heads of
-// D.  A wave a head: the sum of squares stays in the wave.
+// D.  A wave a head: the sum of squares stays in the wave; a block takes four heads of a row
+// (grid: rows x groups of four heads).
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(AP_THREADS) void head_norm_rotate_store_kernel(
@@ -423,7 +424,7 @@ __global__ __launch_bounds__(AP_THREADS) void head_norm_rotate_store_kernel(
   const int slot = pos % ps;
   if (k_pool != nullptr) page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
   // heads 0 .. H - 1 are queries, H .. H + G - 1 keys, then the G value heads
-  for (int head = wave; head < H + 2 * G; head += NW) {
+  for (int head = blockIdx.y * NW + wave; head < H + 2 * G; head += gridDim.y * NW) {
     if (head >= H + G) {
       if (k_pool == nullptr) continue;
       const int g = head - H - G;
@@ -466,6 +467,81 @@ __global__ __launch_bounds__(AP_THREADS) void head_norm_rotate_store_kernel(
   }
 }
 
+// The same for bfloat16 heads whose sizes are multiples of eight: a lane takes eight neighbouring
+// places of a head (16-byte loads and stores), D / 8 lanes a head (a power of two), several heads
+// a wave; sums of squares and rotation partners travel between lanes, not through memory.  The
+// rotation pairs place i with i + rot_dims / 2, and rot_dims / 2 is a multiple of eight (or
+// nothing turns).
+template <int LPH>
+__global__ __launch_bounds__(AP_THREADS) void head_norm_rotate_store_vec_kernel(
+    const bf16_t* __restrict__ proj, int stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rot_dims, bf16_t* __restrict__ k_pool,
+    bf16_t* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int dv, int D,
+    int ps, bf16_t* __restrict__ q_out) {
+  constexpr int HPW = WAVE / LPH, NW = AP_THREADS / WAVE;
+  const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int head = (blockIdx.y * NW + wave) * HPW + lane / LPH, sub = lane % LPH, e0 = sub * 8;
+  const int n_heads = H + 2 * G;
+  const bool live = head < n_heads && e0 < D && (head < H || k_pool != nullptr);
+  const int pos = row_pos[t];
+  const bf16_t* row = proj + (size_t)t * stride;
+  const int nq = H * d, nk = G * d, half = rot_dims / 2;
+  const bool is_v = head >= H + G, is_q = head < H;
+  const int width = is_v ? dv : d;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = 0.f;
+  if (live && e0 < width) {
+    const bf16_t* src = is_q ? row + head * d : is_v ? row + nq + nk + (head - H - G) * dv
+                                                     : row + nq + (head - H) * d;
+    load8(src + e0, v);
+  }
+  const float* w = is_q ? q_norm_w : k_norm_w;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+#pragma unroll
+  for (int m = 1; m < LPH; m *= 2) ss += __shfl_xor(ss, m);
+  if (!is_v && w != nullptr && live && e0 < d) {
+    const float r = 1.0f / sqrtf(ss / (float)d + eps);
+    float wv[8];
+    load8(w + e0, wv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] *= r * wv[i];
+  }
+  // rotation partners: the lane half / 8 further on (first half) or back (second half)
+  const bool turns = !is_v && rot_dims > 0 && e0 < rot_dims;
+  const bool first = e0 < half;
+  const int partner = turns ? (first ? lane + half / 8 : lane - half / 8) : lane;
+  float pv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) pv[i] = __shfl(v[i], partner);
+  if (turns && live) {
+    const int j0 = first ? e0 : e0 - half;
+    float c[8], sn[8];
+    load8(cos_tab + (size_t)pos * half + j0, c);
+    load8(sin_tab + (size_t)pos * half + j0, sn);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = first ? v[i] * c[i] - pv[i] * sn[i] : v[i] * c[i] + pv[i] * sn[i];
+  }
+  if (!live) return;
+  if (is_q) {
+    store8(q_out + ((size_t)t * H + head) * D + e0, v);
+    return;
+  }
+  const size_t page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
+  const int slot = pos % ps;
+  if (!is_v) {
+    store8(k_pool + ((page * G + (head - H)) * ps + slot) * D + e0, v);
+  } else {
+    bf16_t* dst = v_pool + ((page * G + (head - H - G)) * D + e0) * ps + slot;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[(size_t)i * ps] = f32_to_bf16(v[i]);
+  }
+}
+
 extern "C" int kappai_head_norm_rotate_store(
     const void* proj, int stride, const float* q_norm_w, const float* k_norm_w, float eps,
     const float* cos_tab, const float* sin_tab, int rot_dims, int rot_mode, void* k_pool,
@@ -478,13 +554,40 @@ extern "C" int kappai_head_norm_rotate_store(
       (rot_mode && rot_dims && (!cos_tab || !sin_tab)))
     return (int)hipErrorInvalidValue;
   if (rot_dims == 0) rot_mode = 0;
+  const int lph = D / 8, half = rot_dims / 2;
+  if (is_bf16 && d % 8 == 0 && dv % 8 == 0 && D % 8 == 0 && stride % 8 == 0 &&
+      (uintptr_t)proj % 16 == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_pool % 16 == 0 &&
+      (lph == 1 || lph == 2 || lph == 4 || lph == 8 || lph == 16 || lph == 32) &&
+      (rot_mode == 0 || (rot_mode == 1 && half % 8 == 0)) &&
+      (!q_norm_w || (uintptr_t)q_norm_w % 16 == 0) && (!k_norm_w || (uintptr_t)k_norm_w % 16 == 0) &&
+      (rot_mode == 0 || (((uintptr_t)cos_tab | (uintptr_t)sin_tab) % 16 == 0))) {
+    const int per_block = (AP_THREADS / WAVE) * (WAVE / lph);
+    const dim3 grid(T, (H + 2 * G + per_block - 1) / per_block);
+    if (grid.y > 65535) return (int)hipErrorInvalidValue;
+#define HNRS_VEC(L)                                                                              \
+  hipLaunchKernelGGL(head_norm_rotate_store_vec_kernel<L>, grid, dim3(AP_THREADS), 0, stream,     \
+                     (const bf16_t*)proj, stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,      \
+                     rot_mode ? rot_dims : 0, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg, \
+                     block_tables, max_blocks, H, G, d, dv, D, ps, (bf16_t*)q_out)
+    switch (lph) {
+      case 1: HNRS_VEC(1); break;
+      case 2: HNRS_VEC(2); break;
+      case 4: HNRS_VEC(4); break;
+      case 8: HNRS_VEC(8); break;
+      case 16: HNRS_VEC(16); break;
+      default: HNRS_VEC(32); break;
+    }
+#undef HNRS_VEC
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
+  const dim3 hn_grid(T, min(65535, (H + 2 * G + AP_THREADS / WAVE - 1) / (AP_THREADS / WAVE)));
   if (is_bf16)
-    hipLaunchKernelGGL(head_norm_rotate_store_kernel<bf16_t>, dim3(T), dim3(AP_THREADS), 0,
+    hipLaunchKernelGGL(head_norm_rotate_store_kernel<bf16_t>, hn_grid, dim3(AP_THREADS), 0,
                        stream, (const bf16_t*)proj, stride, q_norm_w, k_norm_w, eps, cos_tab,
                        sin_tab, rot_dims, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos,
                        row_seg, block_tables, max_blocks, H, G, d, dv, D, ps, (bf16_t*)q_out);
   else
-    hipLaunchKernelGGL(head_norm_rotate_store_kernel<float>, dim3(T), dim3(AP_THREADS), 0, stream,
+    hipLaunchKernelGGL(head_norm_rotate_store_kernel<float>, hn_grid, dim3(AP_THREADS), 0, stream,
                        (const float*)proj, stride, q_norm_w, k_norm_w, eps, cos_tab, sin_tab,
                        rot_dims, rot_mode, (float*)k_pool, (float*)v_pool, row_pos, row_seg,
                        block_tables, max_blocks, H, G, d, dv, D, ps, (float*)q_out);

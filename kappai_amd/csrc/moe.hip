@@ -504,7 +504,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(
     const float* __restrict__ wts, int top, int D, const void* __restrict__ also,
     int also_is_bf16, int also_parts, size_t also_plane, float* __restrict__ out) {
   const int t = blockIdx.x;
-  for (int n = threadIdx.x; n < D; n += MOE_THREADS) {
+  for (int n = blockIdx.y * MOE_THREADS + threadIdx.x; n < D; n += gridDim.y * MOE_THREADS) {
     // what every row gets beside its experts (a shared expert's result: rows, or float planes
     // of a product cut over its input dimension, added in order) comes first
     float acc = 0.f;
@@ -526,7 +526,9 @@ extern "C" int kappai_moe_combine(const float* y, const int* slot_of_pair, const
                                   int also_parts, float* out, hipStream_t stream) {
   if (T <= 0) return 0;
   if (also && also_parts < 1) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(MOE_THREADS), 0, stream, y, slot_of_pair,
+  // few rows: a thread a column, so that all its loads are asked for at once
+  const int col_blocks = T <= 512 ? min(64, (D + MOE_THREADS - 1) / MOE_THREADS) : 1;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, col_blocks), dim3(MOE_THREADS), 0, stream, y, slot_of_pair,
                      wts, top, D, also, also_is_bf16, also_parts, (size_t)T * D, out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

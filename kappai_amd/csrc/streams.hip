@@ -14,20 +14,31 @@
 //   activate       out = relu(x)^2 (kind 0)
 #include "common.h"
 
-#define HS_THREADS 256
+#define HS_THREADS 256          // threads of a block when there are rows enough to fill the chip
+#define HS_MAX_THREADS 1024     // with few rows a block is as wide as the row has pieces
 #define HS_MAX_STREAMS 8
 
 // VEC values of an update from column c on: rows of TY, or P float planes [P, T, W] added in order
 template <int VEC>
 __device__ __forceinline__ void update_at(const float* __restrict__ y, int parts, size_t plane,
                                           size_t at, float* v) {
+  // four planes are asked for at once and added in their order (a loop that waits for every
+  // plane before it asks for the next costs a trip to memory a plane)
   if (VEC == 4) {
-    const float4 a = *reinterpret_cast<const float4*>(y + at);
-    v[0] = a.x; v[VEC > 1 ? 1 : 0] = a.y; v[VEC > 2 ? 2 : 0] = a.z; v[VEC > 3 ? 3 : 0] = a.w;
-    for (int p = 1; p < parts; ++p) {
-      const float4 b = *reinterpret_cast<const float4*>(y + (size_t)p * plane + at);
-      v[0] += b.x; v[VEC > 1 ? 1 : 0] += b.y; v[VEC > 2 ? 2 : 0] += b.z; v[VEC > 3 ? 3 : 0] += b.w;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int p0 = 0; p0 < parts; p0 += 4) {
+      float4 b[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        b[j] = p0 + j < parts ? *reinterpret_cast<const float4*>(y + (size_t)(p0 + j) * plane + at)
+                              : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (p0 + j == 0) acc = b[j];
+        else if (p0 + j < parts) { acc.x += b[j].x; acc.y += b[j].y; acc.z += b[j].z; acc.w += b[j].w; }
+      }
     }
+    v[0] = acc.x; v[VEC > 1 ? 1 : 0] = acc.y; v[VEC > 2 ? 2 : 0] = acc.z; v[VEC > 3 ? 3 : 0] = acc.w;
   } else {
     v[0] = y[at];
     for (int p = 1; p < parts; ++p) v[0] += y[(size_t)p * plane + at];
@@ -76,9 +87,10 @@ __device__ __forceinline__ void store_rows(bf16_t* p, const float* v) {
 }
 
 // A block a row; a thread takes VEC neighbouring columns at a time (VEC 4: 16-byte loads and
-// stores; the width and every address then are multiples of four values).
-template <typename TY, typename TO, int VEC>
-__global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
+// stores; the width and every address then are multiples of four values).  The weights among the
+// copies go through LDS once a block.
+template <typename TY, typename TO, int VEC, int MAXT>
+__global__ __launch_bounds__(MAXT) void hyper_step_kernel(
     float* __restrict__ streams, const float* __restrict__ source, const TY* __restrict__ y,
     int parts, const float* __restrict__ mix, const float* __restrict__ out_w,
     const float* __restrict__ in_w, const float* __restrict__ norm_w, float eps,
@@ -86,18 +98,22 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   extern __shared__ float hs_lds[];
   float* u_row = hs_lds;                 // [W]
   float* red = hs_lds + W;               // [16]
+  const int t = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const bool write = y != nullptr, read = normed != nullptr;
   __shared__ float c_mix[HS_MAX_STREAMS * HS_MAX_STREAMS], c_out[HS_MAX_STREAMS],
       c_in[HS_MAX_STREAMS];
-  const int t = rows ? rows[blockIdx.x] : blockIdx.x;
-  const int tid = threadIdx.x;
-  if (tid < S * S && mix) c_mix[tid] = mix[tid];
-  if (tid < S && out_w) c_out[tid] = out_w[tid];
-  if (tid < S && in_w) c_in[tid] = in_w[tid];
+  if (tid < S * S && write) c_mix[tid] = mix[tid];
+  if (tid < S && write) c_out[tid] = out_w[tid];
+  if (tid < S && read) c_in[tid] = in_w[tid];
   __syncthreads();
-  const bool write = y != nullptr, read = normed != nullptr;
+  // the norm's weights for this thread's first columns are asked for with the row itself
+  float w_first[VEC];
+  const bool has_first = read && tid * VEC < W;
+  if (has_first) load_f32<VEC>(norm_w + tid * VEC, w_first);
   const size_t plane = (size_t)T * W;
   float sum = 0.f;
-  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+  for (int c = tid * VEC; c < W; c += nthreads * VEC) {
     float x[HS_MAX_STREAMS][VEC];
 #pragma unroll
     for (int s = 0; s < HS_MAX_STREAMS; ++s)
@@ -147,7 +163,7 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   if (!read) return;
   const float mean = block_sum(sum, red) / (float)W;
   float sq = 0.f;
-  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+  for (int c = tid * VEC; c < W; c += nthreads * VEC) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const float d = u_row[c + i] - mean;
@@ -156,9 +172,14 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   }
   const float rstd = 1.0f / sqrtf(block_sum(sq, red) / (float)W + eps);
   TO* dst = normed + (size_t)blockIdx.x * W;
-  for (int c = tid * VEC; c < W; c += HS_THREADS * VEC) {
+  for (int c = tid * VEC; c < W; c += nthreads * VEC) {
     float o[VEC], w[VEC];
-    load_f32<VEC>(norm_w + c, w);
+    if (c == tid * VEC) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) w[i] = w_first[i];
+    } else {
+      load_f32<VEC>(norm_w + c, w);
+    }
 #pragma unroll
     for (int i = 0; i < VEC; ++i) o[i] = (u_row[c + i] - mean) * rstd * w[i];
     store_rows<VEC>(dst + c, o);
@@ -180,12 +201,23 @@ extern "C" int kappai_hyper_step(float* streams, const float* source, const void
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
   const bool vec = W % 4 == 0 && ((uintptr_t)streams | (uintptr_t)source | (uintptr_t)norm_w |
                                   (uintptr_t)normed) % 16 == 0 && (uintptr_t)y % 16 == 0;
-#define HS_LAUNCH_V(TY, TO, V)                                                                   \
-  hipLaunchKernelGGL((hyper_step_kernel<TY, TO, V>), dim3(blocks), dim3(HS_THREADS), lds, stream, \
+  // few rows: every piece of the row has a thread of its own, so all its loads are asked for at
+  // once (a step of single tokens waits for memory, not for bandwidth)
+  int threads = HS_THREADS;
+  if (blocks <= 512) {
+    const int pieces = (W + (vec ? 4 : 1) - 1) / (vec ? 4 : 1);
+    threads = min(HS_MAX_THREADS, max(WAVE, (pieces + WAVE - 1) / WAVE * WAVE));
+  }
+#define HS_LAUNCH_V(TY, TO, V, MT)                                                               \
+  hipLaunchKernelGGL((hyper_step_kernel<TY, TO, V, MT>), dim3(blocks), dim3(threads), lds, stream, \
                      streams, source, (const TY*)y, parts, mix, out_w, in_w, norm_w, eps, rows,   \
                      store, (TO*)normed, T, S, W)
 #define HS_LAUNCH(TY, TO)                                                                        \
-  if (vec) HS_LAUNCH_V(TY, TO, 4); else HS_LAUNCH_V(TY, TO, 1)
+  if (threads > HS_THREADS) {                                                                    \
+    if (vec) HS_LAUNCH_V(TY, TO, 4, HS_MAX_THREADS); else HS_LAUNCH_V(TY, TO, 1, HS_MAX_THREADS); \
+  } else {                                                                                       \
+    if (vec) HS_LAUNCH_V(TY, TO, 4, HS_THREADS); else HS_LAUNCH_V(TY, TO, 1, HS_THREADS);         \
+  }
   if (y_is_bf16) {
     if (normed_is_bf16) { HS_LAUNCH(bf16_t, bf16_t); } else { HS_LAUNCH(bf16_t, float); }
   } else {
@@ -196,21 +228,21 @@ extern "C" int kappai_hyper_step(float* streams, const float* source, const void
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
-// A wave a row: the first n columns of a row of `x` (stride ldx), normed into `out` [T, n].
+// A block a row: the first n columns of a row of `x` (stride ldx), normed into `out` [T, n].
 template <typename T>
 __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(
-    const T* __restrict__ x, int ldx, const float* __restrict__ w, float eps, int n_rows, int n,
+    const T* __restrict__ x, int ldx, const float* __restrict__ w, float eps, int n,
     T* __restrict__ out) {
-  const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  if (row >= n_rows) return;
+  __shared__ float red[16];
+  const int row = blockIdx.x;
   const T* xr = x + (size_t)row * ldx;
   float sq = 0.f;
-  for (int c = lane; c < n; c += WAVE) {
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
     const float v = to_f32(xr[c]);
     sq = fmaf(v, v, sq);
   }
-  const float r = 1.0f / sqrtf(wave_sum(sq) / (float)n + eps);
-  for (int c = lane; c < n; c += WAVE)
+  const float r = 1.0f / sqrtf(block_sum(sq, red) / (float)n + eps);
+  for (int c = threadIdx.x; c < n; c += blockDim.x)
     from_f32(out + (size_t)row * n + c, to_f32(xr[c]) * r * w[c]);
 }
 
@@ -218,13 +250,13 @@ extern "C" int kappai_rows_rmsnorm(const void* x, int ldx, const float* w, float
                                    int n, void* out, int is_bf16, hipStream_t stream) {
   if (T <= 0) return 0;
   if (n < 1 || ldx < n) return (int)hipErrorInvalidValue;
-  const dim3 grid((T + 3) / 4), block(256);
+  const dim3 grid(T), block(n <= 64 ? 64 : n <= 128 ? 128 : 256);
   if (is_bf16)
     hipLaunchKernelGGL(rows_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, ldx,
-                       w, eps, T, n, (bf16_t*)out);
+                       w, eps, n, (bf16_t*)out);
   else
     hipLaunchKernelGGL(rows_rmsnorm_kernel<float>, grid, block, 0, stream, (const float*)x, ldx, w,
-                       eps, T, n, (float*)out);
+                       eps, n, (float*)out);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
