@@ -133,7 +133,7 @@ class LayerNorm(Norm):
                 eps=self.eps, rows=rows, rows_dtype=self.dtype)
 
     def add_norm(self, resid, delta, rows=None):
-        """The ``Norm`` contract on one stream [T, width]; or, on a stream in copies [T, S, width]
+        """The ``Norm`` interface on one stream [T, width]; or, on a stream in copies [T, S, width]
         with a pending ``StreamUpdate`` (or None), the norm of the copies' plain sum."""
         if isinstance(delta, ops.Added):
             delta = None

@@ -128,7 +128,7 @@ def test_one_pass_over_the_copies_of_the_stream(S, W):
     assert rel(rows, normed[pick.long()]) < 2e-5
 
 
-def test_layer_norm_part_keeps_the_norm_contract():
+def test_layer_norm_part_keeps_the_norm_interface():
     """On one stream [T, width]: the pending update is added in float32 and the rows normalised;
     with ``rows`` the stream stays as it is."""
     from kappai_amd.parts import LayerNorm
