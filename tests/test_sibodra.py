@@ -21,9 +21,10 @@ from kappai_amd.config.sibodra import SibodraConfig
 from kappai_amd.engine.replay import TraceReplayer, make_replay_cache
 from kappai_amd.models import build_model, load_model
 
-LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [40, 75]}
+LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [40, 75], "E": [61, 30, 45]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58], "B": [66, 35, 90, 41, 23, 77, 50, 62, 88],
-                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [40, 75, 52, 33, 61, 28]}
+                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [40, 75, 52, 33, 61, 28],
+                 "E": [61, 30, 45, 38, 52, 27, 66]}
 
 
 @pytest.fixture(scope="module")
@@ -181,7 +182,8 @@ def run_emulated(monkeypatch, model_dir, steps, index, max_tokens, tmp_path):
 @pytest.mark.parametrize("name,family", [("A", f) for f in
                                          ("whole", "prefill_then_decode", "changing_portions",
                                           "mixed")] + [("B", "mixed"), ("C", "mixed"),
-                                                       ("D", "changing_portions")])
+                                                       ("D", "changing_portions"),
+                                                       ("E", "mixed")])
 def test_schedules_float32(monkeypatch, tmp_path, model_dirs, name, family):
     cfg = TINY[name][0]
     lengths = MIXED_LENGTHS[name] if family == "mixed" else LENGTHS[name]

@@ -20,9 +20,10 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 F32, BF16, F64 = torch.float32, torch.bfloat16, torch.float64
 
-LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [40, 75, 130]}
+LENGTHS = {"A": [70, 45, 100, 37], "B": [66, 35, 90], "C": [50, 81, 36], "D": [40, 75, 130], "E": [61, 30, 45]}
 MIXED_LENGTHS = {"A": [70, 45, 100, 37, 83, 64, 29, 58], "B": [66, 35, 90, 41, 23, 77, 50, 62, 88],
-                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [40, 75, 52, 33, 61, 28, 97]}
+                 "C": [50, 81, 36, 67, 44, 72, 90, 33, 58], "D": [40, 75, 52, 33, 61, 28, 97],
+                 "E": [61, 30, 45, 38, 52, 27, 66]}
 
 
 def gen(seed):
@@ -65,7 +66,7 @@ PORTIONS_150 = [37, 3] + [1] * 50 + [2, 33] + [1] * 25
 # kernels alone
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("S", [1, 2, 3, 4, 8])
-@pytest.mark.parametrize("W", [72, 64, 328, 2048, 100])
+@pytest.mark.parametrize("W", [72, 64, 328, 2048, 100, 67, 30])
 def test_one_pass_over_the_copies_of_the_stream(S, W):
     """Update, weighted sum and layer norm in one kernel, against their formulas in float64: the
     update as float32 rows, bfloat16 rows and float32 partial sums; the read half alone; the write
@@ -424,7 +425,7 @@ def replay(model_dir, dtype, steps, index, max_tokens, out_dir, slots=4, graphs=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     """Every logit of every request.  The mixed family runs in a pool smaller than its requests

@@ -88,8 +88,16 @@ TINY_D = config(500, 100, 1e-5, 4, 25.0, [
 ])
 INIT_D = dict(seed=44, std=0.08, norm_jitter=0.1)
 
+# a width, a vocabulary and head sizes that are multiples of nothing: no kernel takes 16 bytes at
+# a time here; two copies of the stream
+TINY_E = config(131, 54, 1e-5, 2, 9.0, [
+    latent(3, 10, 6, 14, 11, 9, 0.22, 777.0, moe(10, 5, 2, shared=6)),
+    attention(3, 1, 10, 6, 0.3, 6.0, 1234.0, 4, (3.0, 1.0, 3.0, 16), dense(34)),
+])
+INIT_E = dict(seed=45, std=0.2, norm_jitter=0.1)
+
 TINY = {"A": (TINY_A, INIT_A), "B": (TINY_B, INIT_B), "C": (TINY_C, INIT_C),
-        "D": (TINY_D, INIT_D)}
+        "D": (TINY_D, INIT_D), "E": (TINY_E, INIT_E)}
 
 
 def write_tiny(name: str, folder, **overrides):
