@@ -4,8 +4,8 @@
 //   hyper_step     one pass over a row's S copies x_1 .. x_S [T, S, W] (float32):
 //                    write:  x_t <- sum_s mix[s, t] x_s + out[t] * y     (all t from the old x_s)
 //                    read:   u = sum_s in[s] x_s;  rows = (u - mean) / sqrt(var + eps) * w
-//                  either half may be left out; `spread`: the copies do not exist yet and are all
-//                  the row of `source` [T, W] (the embedded rows); `rows`: only the listed rows
+//                  either half may be left out; `source`: the copies do not exist yet and are all
+//                  that row [T, W] (the embedded rows); `rows`: only the listed rows
 //                  are read (and, with a write half, their new copies are not stored: the norm
 //                  before the output head).
 //   rows_rmsnorm   y = x / sqrt(mean(x^2) + eps) * w on the first n columns of strided rows
